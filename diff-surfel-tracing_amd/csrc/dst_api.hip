@@ -1,0 +1,145 @@
+// C ABI of libdst.so: context management, argument validation, launches.
+// Replaces the pybind module and host launcher of the reference (ext.cpp, trace_surfels.cpp).
+#include "dst_internal.h"
+
+#include <cstring>
+#include <new>
+
+namespace {
+
+const char *kNoCtx = "null context";
+
+int check_common(dst_ctx *ctx, const DstParams *p) {
+    if (!p) return dst_fail(ctx, DST_E_INVALID, "params is null");
+    if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "build_acceleration_structure has not been called");
+    if (p->P <= 0) return dst_fail(ctx, DST_E_INVALID, "means3D must have dimensions (num_points, 3)");
+    if ((uint32_t)p->P != ctx->n_leaves)
+        return dst_fail(ctx, DST_E_INVALID, "number of surfels differs from the acceleration structure (" +
+                                                std::to_string(p->P) + " vs " + std::to_string(ctx->n_leaves) + ")");
+    if (p->H < 0 || p->W < 0) return dst_fail(ctx, DST_E_INVALID, "negative ray grid size");
+    if (p->aux < 1 || p->aux > DST_MAX_AUX)
+        return dst_fail(ctx, DST_E_UNSUPPORTED, "aux channels must be in 1.." + std::to_string(DST_MAX_AUX));
+    if (p->mtd_alloc < 0 || p->mtd_alloc > DST_MAX_TRACE_DEPTH)
+        return dst_fail(ctx, DST_E_UNSUPPORTED, "mtd_alloc must be in 0.." + std::to_string(DST_MAX_TRACE_DEPTH));
+    if (p->max_trace_depth < 0 || p->max_trace_depth > p->mtd_alloc)
+        return dst_fail(ctx, DST_E_INVALID, "max_trace_depth exceeds the depth mid_val was allocated for");
+    if ((p->shs == nullptr) == (p->colors_precomp == nullptr))
+        return dst_fail(ctx, DST_E_INVALID, "exactly one of shs / colors_precomp must be given");
+    if (p->shs && (p->D < 0 || p->D > 3 || (p->D + 1) * (p->D + 1) > p->M))
+        return dst_fail(ctx, DST_E_INVALID, "sh_degree must be 0..3 and fit the coefficients in shs");
+    if (p->H > 0 && p->W > 0 && (!p->ray_o || !p->ray_d))
+        return dst_fail(ctx, DST_E_INVALID, "ray_o / ray_d missing");
+    if (!p->vertices || !p->background || !p->means3D || !p->opacities || !p->scales || !p->rotations)
+        return dst_fail(ctx, DST_E_INVALID,
+                        "vertices, background, means3D, opacities, scales and rotations are required");
+    if (p->H > 0 && p->W > 0 &&
+        (!p->out_rgb || !p->out_dpt || !p->out_acc || !p->out_norm || !p->out_dist || !p->out_aux || !p->mid_val))
+        return dst_fail(ctx, DST_E_INVALID, "forward output buffers missing");
+    return DST_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *dst_version(void) { return "dst-mi355x 0.1"; }
+size_t dst_sizeof_params(void) { return sizeof(DstParams); }
+
+dst_ctx *dst_create(void) {
+    dst_ctx *ctx = new (std::nothrow) dst_ctx();
+    if (!ctx) return nullptr;
+    if (hipGetDevice(&ctx->device) != hipSuccess) {
+        delete ctx;
+        return nullptr;
+    }
+    return ctx;
+}
+
+void dst_destroy(dst_ctx *ctx) {
+    if (!ctx) return;
+    dst_lbvh_free(ctx);
+    if (ctx->bounds) (void)hipFree(ctx->bounds);
+    if (ctx->bounds_host) (void)hipHostFree(ctx->bounds_host);
+    delete ctx;
+}
+
+const char *dst_last_error(dst_ctx *ctx) { return ctx ? ctx->err.c_str() : kNoCtx; }
+
+int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
+                    uint32_t n_triangles, int rebuild, void *stream) {
+    if (!ctx) return DST_E_INVALID;
+    if (!vertices) return dst_fail(ctx, DST_E_INVALID, "vertices must have dimensions (num_vertices, 3)");
+    if (n_triangles == 0 || (n_triangles & 1u))
+        return dst_fail(ctx, DST_E_TOPOLOGY, "triangles must have dimensions (2 * num_surfels, 3)");
+    const uint32_t P = n_triangles / 2;
+    if ((uint64_t)n_vertices < 4ull * P)
+        return dst_fail(ctx, DST_E_TOPOLOGY, "vertices must hold four corners per surfel (4 * num_surfels, 3)");
+    if (P > 0x7FFFFFFFu / 4u) return dst_fail(ctx, DST_E_UNSUPPORTED, "too many surfels");
+    if (rebuild) {
+        if (!triangles) return dst_fail(ctx, DST_E_INVALID, "triangles must have dimensions (num_triangles, 3)");
+    } else {
+        if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "refit (rebuild=False) before any build");
+        if (P != ctx->n_leaves)
+            return dst_fail(ctx, DST_E_TOPOLOGY, "refit (rebuild=False) with a different number of surfels");
+    }
+    return dst_lbvh_build(ctx, vertices, n_vertices, triangles, P, rebuild != 0, (hipStream_t)stream);
+}
+
+int dst_trace_forward(dst_ctx *ctx, const DstParams *p, void *stream) {
+    if (!ctx) return DST_E_INVALID;
+    int rc = check_common(ctx, p);
+    if (rc) return rc;
+    if (p->training && !p->a_weights) return dst_fail(ctx, DST_E_INVALID, "training needs a_weights");
+    return dst_launch_trace(ctx, *p, false, (hipStream_t)stream);
+}
+
+int dst_trace_backward(dst_ctx *ctx, const DstParams *p, void *stream) {
+    if (!ctx) return DST_E_INVALID;
+    int rc = check_common(ctx, p);
+    if (rc) return rc;
+    if (p->H > 0 && p->W > 0 &&
+        (!p->dL_drgb || !p->dL_ddpt || !p->dL_dacc || !p->dL_dnorm || !p->dL_daux || !p->dL_dray_o || !p->dL_dray_d))
+        return dst_fail(ctx, DST_E_INVALID, "upstream gradients or ray gradient buffers missing");
+    if (!p->dL_dmeans3D || !p->dL_dgrads3D || !p->dL_dcolors || !p->dL_dopacities || !p->dL_dscales ||
+        !p->dL_drotations)
+        return dst_fail(ctx, DST_E_INVALID, "per-surfel gradient buffers missing");
+    if (p->shs && !p->dL_dshs) return dst_fail(ctx, DST_E_INVALID, "dL_dshs missing");
+    if (p->others_precomp && !p->dL_dothers) return dst_fail(ctx, DST_E_INVALID, "dL_dothers missing");
+    return dst_launch_trace(ctx, *p, true, (hipStream_t)stream);
+}
+
+int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info) {
+    if (!ctx || !info) return DST_E_INVALID;
+    if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "no acceleration structure");
+    info->n_surfels = ctx->n_leaves;
+    info->n_internal = ctx->n_leaves - 1;
+    info->root = (ctx->n_leaves == 1) ? DST_LEAF_BIT : 0u;
+    info->node_bytes = sizeof(DstNode);
+    info->leaf_bytes = sizeof(DstLeaf);
+    for (int a = 0; a < 3; ++a) {
+        info->scene_lo[a] = ctx->scene_lo[a];
+        info->scene_hi[a] = ctx->scene_hi[a];
+    }
+    info->max_abs = ctx->max_abs;
+    info->builds = ctx->builds;
+    info->refits = ctx->refits;
+    return DST_OK;
+}
+
+int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_parent, uint32_t *leaf_parent,
+                       uint32_t *sorted_keys, void *stream) {
+    if (!ctx) return DST_E_INVALID;
+    if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "no acceleration structure");
+    hipStream_t s = (hipStream_t)stream;
+    DST_HIP(ctx, hipStreamSynchronize(s));
+    const size_t n = ctx->n_leaves;
+    if (nodes && n > 1) DST_HIP(ctx, hipMemcpy(nodes, ctx->nodes, sizeof(DstNode) * (n - 1), hipMemcpyDeviceToHost));
+    if (leaves) DST_HIP(ctx, hipMemcpy(leaves, ctx->leaves, sizeof(DstLeaf) * n, hipMemcpyDeviceToHost));
+    if (node_parent && n > 1)
+        DST_HIP(ctx, hipMemcpy(node_parent, ctx->node_parent, sizeof(uint32_t) * (n - 1), hipMemcpyDeviceToHost));
+    if (leaf_parent) DST_HIP(ctx, hipMemcpy(leaf_parent, ctx->leaf_parent, sizeof(uint32_t) * n, hipMemcpyDeviceToHost));
+    if (sorted_keys) DST_HIP(ctx, hipMemcpy(sorted_keys, ctx->keys[0], sizeof(uint32_t) * n, hipMemcpyDeviceToHost));
+    return DST_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+// Internal declarations shared by the BVH builder, the trace kernels and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+
+#include "dst_api.h"
+
+#define DST_LEAF_BIT 0x80000000u
+#define DST_NO_PARENT 0xFFFFFFFFu
+#define DST_WAVE 64
+
+// Internal node of the binary BVH: the boxes of both children live in the parent, so one
+// 64-byte wave-uniform fetch decides both descents.
+struct alignas(64) DstNode {
+    float lo0[3], hi0[3];
+    float lo1[3], hi1[3];
+    uint32_t c0, c1;  // child references: DST_LEAF_BIT | leaf position, or internal node index
+    uint32_t pad[2];
+};
+
+// Leaf = one surfel quad in Morton order: corners A,B,C,D (triangles ABC and BCD) and the surfel id.
+struct alignas(64) DstLeaf {
+    float A[3], B[3], C[3], D[3];
+    uint32_t g;
+    uint32_t pad[3];
+};
+
+struct DstBounds {          // device-resident reduction targets, order-preserving uint encoding
+    uint32_t lo[3], hi[3];  // centroid bounds
+    uint32_t max_abs;       // raw bits of a non-negative float: largest |coordinate| of any vertex
+    uint32_t bad_topology;  // set by the quad set-up kernel
+};
+
+// Device-side view of the acceleration structure handed to the trace kernels.
+struct DstAccelView {
+    const DstNode *nodes;
+    const DstLeaf *leaves;
+    const DstBounds *bounds;  // max_abs sizes the conservative slab padding; read on the device so that a
+                              // refit never needs a host round trip
+    uint32_t root;
+    uint32_t n_leaves;
+};
+
+struct dst_ctx {
+    int device = 0;
+    std::string err;
+    // acceleration structure
+    uint32_t n_leaves = 0;      // surfels in the current structure
+    uint32_t capacity = 0;      // surfels the buffers can hold
+    bool built = false;
+    uint32_t builds = 0, refits = 0;
+    DstNode *nodes = nullptr;
+    DstLeaf *leaves = nullptr;
+    uint32_t *node_parent = nullptr, *leaf_parent = nullptr;  // (parent << 1) | which child
+    uint32_t *flags = nullptr;                                // arrival counters of the bottom-up fit
+    int32_t *quad_ids = nullptr;                              // 4 vertex ids per surfel (int4)
+    float *centroids = nullptr;                               // 4 floats per surfel
+    uint32_t *keys[2] = {nullptr, nullptr}, *vals[2] = {nullptr, nullptr};
+    uint32_t *tile_hist = nullptr;
+    size_t tile_hist_elems = 0;
+    DstBounds *bounds = nullptr;       // device
+    DstBounds *bounds_host = nullptr;  // pinned host copy
+    float scene_lo[3] = {0, 0, 0}, scene_hi[3] = {0, 0, 0}, max_abs = 0;
+};
+
+// lbvh.hip
+int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
+                   uint32_t n_surfels, bool rebuild, hipStream_t stream);
+void dst_lbvh_free(dst_ctx *ctx);
+// trace.hip
+int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream);
+
+static inline int dst_fail(dst_ctx *ctx, int code, const std::string &msg) {
+    if (ctx) ctx->err = msg;
+    return code;
+}
+#define DST_HIP(ctx, call)                                                                       \
+    do {                                                                                         \
+        hipError_t e_ = (call);                                                                  \
+        if (e_ != hipSuccess)                                                                    \
+            return dst_fail(ctx, DST_E_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_)); \
+    } while (0)

@@ -1,0 +1,453 @@
+// LBVH over the surfel quads: Morton codes -> LDS-staged radix sort -> Karras hierarchy ->
+// bottom-up box fit, plus the refit-only path that keeps topology and leaf order.
+// Replaces the OptiX GAS build / update of the reference (trace_surfels.cpp:36-159).
+#include "dst_internal.h"
+
+#include <algorithm>
+#include <cstring>
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kTile = 1024;        // keys per wave in the radix sort
+constexpr int kRadixBits = 8;
+constexpr int kRadix = 1 << kRadixBits;
+
+__device__ __forceinline__ uint32_t f2ord(float f) {
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__host__ __device__ __forceinline__ float ord2f(uint32_t u) {
+    u = (u & 0x80000000u) ? (u & 0x7fffffffu) : ~u;
+#ifdef __HIP_DEVICE_COMPILE__
+    return __uint_as_float(u);
+#else
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+#endif
+}
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+__global__ void k_init_bounds(DstBounds *b) {
+    if (threadIdx.x == 0) {
+        for (int a = 0; a < 3; ++a) { b->lo[a] = 0xFFFFFFFFu; b->hi[a] = 0u; }
+        b->max_abs = 0u;
+        b->bad_topology = 0u;
+    }
+}
+
+__global__ void k_fill_u32(uint32_t *p, uint32_t v, uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// Per surfel: resolve the quad's four vertex ids through the triangle buffer (build) or reuse them
+// (refit), then reduce centroid bounds and the largest |coordinate|.
+template <bool REBUILD>
+__global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vertices,
+                             const int32_t *__restrict__ triangles, int4 *__restrict__ quad_ids,
+                             float4 *__restrict__ centroids, DstBounds *__restrict__ bounds, uint32_t P) {
+    uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
+    float lo[3] = {INFINITY, INFINITY, INFINITY}, hi[3] = {-INFINITY, -INFINITY, -INFINITY};
+    float cen[3] = {INFINITY, INFINITY, INFINITY}, cenh[3] = {-INFINITY, -INFINITY, -INFINITY};
+    float mabs = 0.f;
+    if (g < P) {
+        int4 q;
+        if (REBUILD) {
+            const int32_t *t = triangles + (size_t)g * 6;
+            q = make_int4(t[0], t[1], t[2], t[5]);
+            bool bad = (t[3] != t[1]) || (t[4] != t[2]);
+            bad |= (uint32_t)q.x >= n_vertices || (uint32_t)q.y >= n_vertices || (uint32_t)q.z >= n_vertices ||
+                   (uint32_t)q.w >= n_vertices;
+            if (bad) {
+                atomicOr(&bounds->bad_topology, 1u);
+                q = make_int4(0, 0, 0, 0);
+            }
+            quad_ids[g] = q;
+        } else {
+            q = quad_ids[g];
+        }
+        const int ids[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float *v = vertices + (size_t)ids[k] * 3;
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                float c = v[a];
+                lo[a] = fminf(lo[a], c);
+                hi[a] = fmaxf(hi[a], c);
+                mabs = fmaxf(mabs, fabsf(c));
+            }
+        }
+        float4 c4;
+        c4.x = 0.5f * (lo[0] + hi[0]);
+        c4.y = 0.5f * (lo[1] + hi[1]);
+        c4.z = 0.5f * (lo[2] + hi[2]);
+        c4.w = 0.f;
+        centroids[g] = c4;
+        cen[0] = cenh[0] = c4.x;
+        cen[1] = cenh[1] = c4.y;
+        cen[2] = cenh[2] = c4.z;
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        cen[a] = wave_min(cen[a]);
+        cenh[a] = wave_max(cenh[a]);
+    }
+    mabs = wave_max(mabs);
+    if ((threadIdx.x & (DST_WAVE - 1)) == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            if (cen[a] <= cenh[a]) {  // skips empty and NaN-only waves
+                atomicMin(&bounds->lo[a], f2ord(cen[a]));
+                atomicMax(&bounds->hi[a], f2ord(cenh[a]));
+            }
+        }
+        if (mabs > 0.f && mabs < INFINITY) atomicMax(&bounds->max_abs, __float_as_uint(mabs));
+    }
+}
+
+__device__ __forceinline__ uint32_t spread10(uint32_t v) {
+    v &= 0x3FFu;
+    v = (v | (v << 16)) & 0x030000FFu;
+    v = (v | (v << 8)) & 0x0300F00Fu;
+    v = (v | (v << 4)) & 0x030C30C3u;
+    v = (v | (v << 2)) & 0x09249249u;
+    return v;
+}
+
+__global__ void k_morton(const float4 *__restrict__ centroids, const DstBounds *__restrict__ bounds,
+                         uint32_t *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t P) {
+    uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= P) return;
+    float4 c = centroids[g];
+    const float cc[3] = {c.x, c.y, c.z};
+    uint32_t q[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float lo = ord2f(bounds->lo[a]), hi = ord2f(bounds->hi[a]);
+        float ext = hi - lo;
+        float s = (ext > 0.f && ext < INFINITY) ? 1024.0f / ext : 0.f;
+        float x = (cc[a] - lo) * s;
+        x = fminf(fmaxf(x, 0.f), 1023.f);  // NaN -> 0
+        q[a] = (uint32_t)x;
+    }
+    keys[g] = (spread10(q[0]) << 2) | (spread10(q[1]) << 1) | spread10(q[2]);
+    vals[g] = g;
+}
+
+// ---- radix sort: one wave owns a contiguous tile of kTile keys ------------------------------------
+__global__ void k_radix_hist(const uint32_t *__restrict__ keys, uint32_t *__restrict__ tile_hist, uint32_t n,
+                             uint32_t n_tiles, int shift) {
+    __shared__ uint32_t hist[kBlock / DST_WAVE][kRadix];
+    const int w = threadIdx.x / DST_WAVE, lane = threadIdx.x % DST_WAVE;
+    const uint32_t tile = blockIdx.x * (kBlock / DST_WAVE) + w;
+    for (int d = lane; d < kRadix; d += DST_WAVE) hist[w][d] = 0;
+    __syncthreads();
+    if (tile < n_tiles) {
+        for (int r = 0; r < kTile / DST_WAVE; ++r) {
+            uint32_t i = tile * kTile + r * DST_WAVE + lane;
+            if (i < n) atomicAdd(&hist[w][(keys[i] >> shift) & (kRadix - 1)], 1u);
+        }
+    }
+    __syncthreads();
+    if (tile < n_tiles)
+        for (int d = lane; d < kRadix; d += DST_WAVE) tile_hist[(size_t)d * n_tiles + tile] = hist[w][d];
+}
+
+// Exclusive scan of `len` counters in place, one block.
+__global__ void k_scan_exclusive(uint32_t *data, uint32_t len) {
+    __shared__ uint32_t part[1024];
+    const uint32_t t = threadIdx.x, nt = blockDim.x;
+    const uint32_t per = (len + nt - 1) / nt;
+    const uint32_t b = t * per, e = min(b + per, len);
+    uint32_t s = 0;
+    for (uint32_t i = b; i < e; ++i) s += data[i];
+    part[t] = s;
+    __syncthreads();
+    for (uint32_t off = 1; off < nt; off <<= 1) {
+        uint32_t v = (t >= off) ? part[t - off] : 0;
+        __syncthreads();
+        part[t] += v;
+        __syncthreads();
+    }
+    uint32_t run = part[t] - s;
+    for (uint32_t i = b; i < e; ++i) {
+        uint32_t v = data[i];
+        data[i] = run;
+        run += v;
+    }
+}
+
+__global__ void k_radix_scatter(const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
+                                uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
+                                const uint32_t *__restrict__ tile_hist, uint32_t n, uint32_t n_tiles, int shift) {
+    __shared__ uint32_t base[kBlock / DST_WAVE][kRadix];
+    const int w = threadIdx.x / DST_WAVE, lane = threadIdx.x % DST_WAVE;
+    const uint32_t tile = blockIdx.x * (kBlock / DST_WAVE) + w;
+    if (tile < n_tiles)
+        for (int d = lane; d < kRadix; d += DST_WAVE) base[w][d] = tile_hist[(size_t)d * n_tiles + tile];
+    __syncthreads();
+    if (tile >= n_tiles) return;
+    const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int r = 0; r < kTile / DST_WAVE; ++r) {
+        uint32_t i = tile * kTile + r * DST_WAVE + lane;
+        bool valid = i < n;
+        uint32_t key = valid ? keys_in[i] : 0u, val = valid ? vals_in[i] : 0u;
+        uint32_t digit = (key >> shift) & (kRadix - 1);
+        uint64_t same = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < kRadixBits; ++b) {
+            bool bit = (digit >> b) & 1u;
+            uint64_t bb = __ballot(bit);
+            same &= bit ? bb : ~bb;
+        }
+        uint32_t rank = __popcll(same & lt);
+        uint32_t off = 0;
+        if (valid) off = base[w][digit];
+        if (valid) {
+            keys_out[off + rank] = key;
+            vals_out[off + rank] = val;
+            if (rank == 0) base[w][digit] = off + (uint32_t)__popcll(same);
+        }
+    }
+}
+
+// ---- Karras 2012 hierarchy over the sorted keys -----------------------------------------------------
+__device__ __forceinline__ int delta(const uint32_t *__restrict__ keys, int n, int i, int j) {
+    if (j < 0 || j >= n) return -1;
+    uint32_t a = keys[i], b = keys[j];
+    if (a == b) return 32 + __clz((uint32_t)i ^ (uint32_t)j);
+    return __clz(a ^ b);
+}
+
+__global__ void k_karras(const uint32_t *__restrict__ keys, DstNode *__restrict__ nodes,
+                         uint32_t *__restrict__ node_parent, uint32_t *__restrict__ leaf_parent, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n - 1) return;
+    int d = (delta(keys, n, i, i + 1) - delta(keys, n, i, i - 1)) >= 0 ? 1 : -1;
+    int dmin = delta(keys, n, i, i - d);
+    int lmax = 2;
+    while (delta(keys, n, i, i + lmax * d) > dmin) lmax <<= 1;
+    int l = 0;
+    for (int t = lmax >> 1; t >= 1; t >>= 1)
+        if (delta(keys, n, i, i + (l + t) * d) > dmin) l += t;
+    int j = i + l * d;
+    int dnode = delta(keys, n, i, j);
+    int s = 0;
+    int t = l;
+    do {
+        t = (t + 1) >> 1;
+        if (delta(keys, n, i, i + (s + t) * d) > dnode) s += t;
+    } while (t > 1);
+    int gamma = i + s * d + min(d, 0);
+    int lo = min(i, j), hi = max(i, j);
+    uint32_t c0, c1;
+    if (lo == gamma) {
+        c0 = DST_LEAF_BIT | (uint32_t)gamma;
+        leaf_parent[gamma] = ((uint32_t)i << 1) | 0u;
+    } else {
+        c0 = (uint32_t)gamma;
+        node_parent[gamma] = ((uint32_t)i << 1) | 0u;
+    }
+    if (hi == gamma + 1) {
+        c1 = DST_LEAF_BIT | (uint32_t)(gamma + 1);
+        leaf_parent[gamma + 1] = ((uint32_t)i << 1) | 1u;
+    } else {
+        c1 = (uint32_t)(gamma + 1);
+        node_parent[gamma + 1] = ((uint32_t)i << 1) | 1u;
+    }
+    nodes[i].c0 = c0;
+    nodes[i].c1 = c1;
+    nodes[i].pad[0] = 0;
+    nodes[i].pad[1] = 0;
+    if (i == 0) node_parent[0] = DST_NO_PARENT;
+}
+
+// Leaf records in Morton order (also the whole of a refit's geometry update).
+__global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
+                            const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves, uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t g = sorted_ids[i];
+    int4 q = quad_ids[g];
+    const int ids[4] = {q.x, q.y, q.z, q.w};
+    float out[16];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float *v = vertices + (size_t)ids[k] * 3;
+        out[3 * k + 0] = v[0];
+        out[3 * k + 1] = v[1];
+        out[3 * k + 2] = v[2];
+    }
+    out[12] = __uint_as_float(g);
+    out[13] = out[14] = out[15] = 0.f;
+    float4 *dst = reinterpret_cast<float4 *>(&leaves[i]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
+}
+
+// Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes.
+__global__ void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
+                      const uint32_t *__restrict__ leaf_parent, uint32_t *flags, const DstLeaf *__restrict__ leaves,
+                      uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const DstLeaf &L = leaves[i];
+    float box[6];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        box[a] = fminf(fminf(L.A[a], L.B[a]), fminf(L.C[a], L.D[a]));
+        box[3 + a] = fmaxf(fmaxf(L.A[a], L.B[a]), fmaxf(L.C[a], L.D[a]));
+    }
+    uint32_t pp = leaf_parent[i];
+    while (pp != DST_NO_PARENT) {
+        const uint32_t p = pp >> 1, which = pp & 1u;
+        float *mine = which ? nodes[p].lo1 : nodes[p].lo0;
+        const float *other = which ? nodes[p].lo0 : nodes[p].lo1;
+#pragma unroll
+        for (int k = 0; k < 6; ++k) __hip_atomic_store(mine + k, box[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        uint32_t arrived = atomicAdd(&flags[p], 1u);
+        if (arrived == 0) return;
+        __threadfence();
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            float olo = __hip_atomic_load(other + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            float ohi = __hip_atomic_load(other + 3 + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            box[k] = fminf(box[k], olo);
+            box[3 + k] = fmaxf(box[3 + k], ohi);
+        }
+        pp = node_parent[p];
+    }
+}
+
+inline dim3 grid_for(uint32_t n, int block = kBlock) { return dim3((n + block - 1) / block); }
+
+int ensure_capacity(dst_ctx *ctx, uint32_t P) {
+    if (P <= ctx->capacity) return DST_OK;
+    dst_lbvh_free(ctx);
+    const size_t n = P;
+    const size_t tiles = (n + kTile - 1) / kTile;
+    DST_HIP(ctx, hipMalloc((void **)&ctx->nodes, sizeof(DstNode) * std::max<size_t>(n - 1, 1)));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->leaves, sizeof(DstLeaf) * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->node_parent, sizeof(uint32_t) * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->leaf_parent, sizeof(uint32_t) * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->flags, sizeof(uint32_t) * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->quad_ids, sizeof(int32_t) * 4 * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->centroids, sizeof(float) * 4 * n));
+    for (int k = 0; k < 2; ++k) {
+        DST_HIP(ctx, hipMalloc((void **)&ctx->keys[k], sizeof(uint32_t) * n));
+        DST_HIP(ctx, hipMalloc((void **)&ctx->vals[k], sizeof(uint32_t) * n));
+    }
+    ctx->tile_hist_elems = tiles * kRadix;
+    DST_HIP(ctx, hipMalloc((void **)&ctx->tile_hist, sizeof(uint32_t) * ctx->tile_hist_elems));
+    if (!ctx->bounds) DST_HIP(ctx, hipMalloc((void **)&ctx->bounds, sizeof(DstBounds)));
+    if (!ctx->bounds_host) DST_HIP(ctx, hipHostMalloc((void **)&ctx->bounds_host, sizeof(DstBounds), hipHostMallocDefault));
+    ctx->capacity = P;
+    return DST_OK;
+}
+
+}  // namespace
+
+void dst_lbvh_free(dst_ctx *ctx) {
+    auto rel = [](auto *&p) {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+    };
+    rel(ctx->nodes);
+    rel(ctx->leaves);
+    rel(ctx->node_parent);
+    rel(ctx->leaf_parent);
+    rel(ctx->flags);
+    rel(ctx->quad_ids);
+    rel(ctx->centroids);
+    rel(ctx->keys[0]);
+    rel(ctx->keys[1]);
+    rel(ctx->vals[0]);
+    rel(ctx->vals[1]);
+    rel(ctx->tile_hist);
+    ctx->capacity = 0;
+    ctx->built = false;
+    ctx->n_leaves = 0;
+}
+
+int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles, uint32_t P,
+                   bool rebuild, hipStream_t stream) {
+    if (rebuild) {
+        ctx->built = false;
+        int rc = ensure_capacity(ctx, P);
+        if (rc) return rc;
+        ctx->n_leaves = P;
+    }
+    const uint32_t n = P;
+    int4 *quad_ids = reinterpret_cast<int4 *>(ctx->quad_ids);
+    float4 *centroids = reinterpret_cast<float4 *>(ctx->centroids);
+
+    hipLaunchKernelGGL(k_init_bounds, dim3(1), dim3(64), 0, stream, ctx->bounds);
+    if (rebuild)
+        hipLaunchKernelGGL(k_quad_setup<true>, grid_for(n), dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
+                           quad_ids, centroids, ctx->bounds, n);
+    else
+        hipLaunchKernelGGL(k_quad_setup<false>, grid_for(n), dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
+                           quad_ids, centroids, ctx->bounds, n);
+
+    if (rebuild) {
+        hipLaunchKernelGGL(k_morton, grid_for(n), dim3(kBlock), 0, stream, centroids, ctx->bounds, ctx->keys[0],
+                           ctx->vals[0], n);
+        const uint32_t tiles = (n + kTile - 1) / kTile;
+        const uint32_t tile_blocks = (tiles + (kBlock / DST_WAVE) - 1) / (kBlock / DST_WAVE);
+        int src = 0;
+        for (int shift = 0; shift < 32; shift += kRadixBits) {
+            hipLaunchKernelGGL(k_radix_hist, dim3(tile_blocks), dim3(kBlock), 0, stream, ctx->keys[src], ctx->tile_hist,
+                               n, tiles, shift);
+            hipLaunchKernelGGL(k_scan_exclusive, dim3(1), dim3(1024), 0, stream, ctx->tile_hist, tiles * kRadix);
+            hipLaunchKernelGGL(k_radix_scatter, dim3(tile_blocks), dim3(kBlock), 0, stream, ctx->keys[src],
+                               ctx->vals[src], ctx->keys[1 - src], ctx->vals[1 - src], ctx->tile_hist, n, tiles, shift);
+            src = 1 - src;
+        }
+        // four passes: the sorted pairs are back in buffer 0
+        if (n > 1) {
+            hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->node_parent, DST_NO_PARENT, n);
+            hipLaunchKernelGGL(k_karras, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->keys[0], ctx->nodes,
+                               ctx->node_parent, ctx->leaf_parent, (int)n);
+        } else {
+            hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(kBlock), 0, stream, ctx->leaf_parent, DST_NO_PARENT, 1u);
+        }
+    }
+    hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0], ctx->leaves,
+                       n);
+    hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->flags, 0u, n);
+    hipLaunchKernelGGL(k_fit, grid_for(n), dim3(kBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
+                       ctx->flags, ctx->leaves, n);
+    DST_HIP(ctx, hipGetLastError());
+
+    if (rebuild) {
+        DST_HIP(ctx, hipMemcpyAsync(ctx->bounds_host, ctx->bounds, sizeof(DstBounds), hipMemcpyDeviceToHost, stream));
+        DST_HIP(ctx, hipStreamSynchronize(stream));
+        if (ctx->bounds_host->bad_topology)
+            return dst_fail(ctx, DST_E_TOPOLOGY,
+                            "triangles must come in pairs [a,b,c],[b,c,d] per surfel with ids inside vertices");
+        for (int a = 0; a < 3; ++a) {
+            ctx->scene_lo[a] = ord2f(ctx->bounds_host->lo[a]);
+            ctx->scene_hi[a] = ord2f(ctx->bounds_host->hi[a]);
+        }
+        std::memcpy(&ctx->max_abs, &ctx->bounds_host->max_abs, 4);
+        ctx->built = true;
+        ctx->builds++;
+    } else {
+        ctx->refits++;
+    }
+    return DST_OK;
+}

@@ -1,0 +1,794 @@
+// Forward trace and backward re-trace kernels.
+//
+// One wavefront (64 lanes) carries an 8x8 tile of rays as a PACKET: the BVH walk is wave-uniform
+// (node and leaf records are fetched once per wave through the scalar path, the traversal stack
+// is a single VGPR indexed by lane), every lane tests its own ray against the shared node / quad,
+// and each lane keeps its own 16-entry nearest-hit buffer in registers.  Replaces the raygen /
+// any-hit programs of the reference (optix_tracer/forward.cu, optix_tracer/backward.cu).
+//
+// Arithmetic that feeds a decision (hit test, hit order, uv, alpha, transmittance, reflection)
+// is plain fp32 evaluated as written: this file is compiled with -ffp-contract=off, rsqrt is
+// 1/sqrt with IEEE division and square root, and exp is the fixed polynomial below.  Only the
+// gradient algebra, which feeds no decision, allows fused multiply-adds.
+#include "dst_internal.h"
+
+namespace {
+
+constexpr int kChunk = 16;
+constexpr float kInfDepth = 1e16f;
+constexpr double kStepEps = 0.00001;
+constexpr int kMaxContrib = 256;
+constexpr float kStartOffset = 0.06f;
+constexpr float kNear = 0.2f;
+constexpr float kTmin = 0.0001f;
+constexpr int kWavesPerBlock = 4;
+
+__device__ const float SH0 = 0.28209479177387814f;
+__device__ const float SH1 = 0.4886025119029199f;
+__device__ const float SH2[5] = {1.0925484305920792f, -1.0925484305920792f, 0.31539156525252005f,
+                                 -1.0925484305920792f, 0.5462742152960396f};
+__device__ const float SH3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.4570457994644658f,
+                                 0.3731763325901154f, -0.4570457994644658f, 1.445305721320277f,
+                                 -0.5900435899266435f};
+
+struct F3 { float x, y, z; };
+__device__ __forceinline__ F3 f3(float x, float y, float z) { return F3{x, y, z}; }
+__device__ __forceinline__ F3 operator+(F3 a, F3 b) { return F3{a.x + b.x, a.y + b.y, a.z + b.z}; }
+__device__ __forceinline__ F3 operator-(F3 a, F3 b) { return F3{a.x - b.x, a.y - b.y, a.z - b.z}; }
+__device__ __forceinline__ F3 operator-(F3 a) { return F3{-a.x, -a.y, -a.z}; }
+__device__ __forceinline__ F3 operator*(F3 a, float s) { return F3{a.x * s, a.y * s, a.z * s}; }
+__device__ __forceinline__ F3 operator*(float s, F3 a) { return F3{s * a.x, s * a.y, s * a.z}; }
+__device__ __forceinline__ F3 operator/(F3 a, float s) { return F3{a.x / s, a.y / s, a.z / s}; }
+__device__ __forceinline__ float dot(F3 a, F3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+__device__ __forceinline__ F3 cross(F3 a, F3 b) {
+    return F3{a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
+}
+__device__ __forceinline__ float length(F3 a) { return __builtin_sqrtf(dot(a, a)); }
+__device__ __forceinline__ F3 ld3(const float *p) { return F3{p[0], p[1], p[2]}; }
+
+// exp for x <= 0 (any x works): Cody-Waite reduction, degree-6 polynomial, exponent patched in.
+__device__ __forceinline__ float exp_det(float x) {
+    if (!(x >= -87.0f)) return 0.0f;
+    if (x > 88.0f) x = 88.0f;
+    float kf = __builtin_rintf(x * 1.44269504088896341f);
+    float r = (x - kf * 0.693359375f) - kf * -2.12194440e-4f;
+    float z = r * r;
+    float p = 1.9875691500e-4f;
+    p = p * r + 1.3981999507e-3f;
+    p = p * r + 8.3334519073e-3f;
+    p = p * r + 4.1665795894e-2f;
+    p = p * r + 1.6666665459e-1f;
+    p = p * r + 5.0000001201e-1f;
+    p = p * z + r;
+    p = p + 1.0f;
+    return __uint_as_float(__float_as_uint(p) + ((uint32_t)((int32_t)kf << 23)));
+}
+
+// quaternion (w,x,y,z) -> rows: tangent u, tangent v, normal (reference auxiliary.h:403-429)
+__device__ __forceinline__ void quat_rows(const float q0, const float q1, const float q2, const float q3, F3 (&R)[3]) {
+    float s = 1.0f / __builtin_sqrtf(q3 * q3 + q0 * q0 + q1 * q1 + q2 * q2);
+    float w = q0 * s, x = q1 * s, y = q2 * s, z = q3 * s;
+    R[0] = f3(1.f - 2.f * (y * y + z * z), 2.f * (x * y + w * z), 2.f * (x * z - w * y));
+    R[1] = f3(2.f * (x * y - w * z), 1.f - 2.f * (x * x + z * z), 2.f * (y * z + w * x));
+    R[2] = f3(2.f * (x * z + w * y), 2.f * (y * z - w * x), 1.f - 2.f * (x * x + y * y));
+}
+
+// SH colour of one surfel in direction d (reference forward.cu:18-58); clamp flags for backward.
+__device__ __forceinline__ F3 sh_color(int deg, const float *__restrict__ sh, F3 d, bool (&neg)[3]) {
+#define SHC(j) f3(sh[3 * (j)], sh[3 * (j) + 1], sh[3 * (j) + 2])
+    F3 r = SH0 * SHC(0);
+    if (deg > 0) {
+        float x = d.x, y = d.y, z = d.z;
+        r = r - SH1 * y * SHC(1) + SH1 * z * SHC(2) - SH1 * x * SHC(3);
+        if (deg > 1) {
+            float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+            r = r + SH2[0] * xy * SHC(4) + SH2[1] * yz * SHC(5) + SH2[2] * (2.0f * zz - xx - yy) * SHC(6) +
+                SH2[3] * xz * SHC(7) + SH2[4] * (xx - yy) * SHC(8);
+            if (deg > 2) {
+                r = r + SH3[0] * y * (3.0f * xx - yy) * SHC(9) + SH3[1] * xy * z * SHC(10) +
+                    SH3[2] * y * (4.0f * zz - xx - yy) * SHC(11) +
+                    SH3[3] * z * (2.0f * zz - 3.0f * xx - 3.0f * yy) * SHC(12) +
+                    SH3[4] * x * (4.0f * zz - xx - yy) * SHC(13) + SH3[5] * z * (xx - yy) * SHC(14) +
+                    SH3[6] * x * (xx - 3.0f * yy) * SHC(15);
+            }
+        }
+    }
+    r = f3(r.x + 0.5f, r.y + 0.5f, r.z + 0.5f);
+    neg[0] = r.x < 0.f;
+    neg[1] = r.y < 0.f;
+    neg[2] = r.z < 0.f;
+    return f3(r.x > 0.f ? r.x : 0.f, r.y > 0.f ? r.y : 0.f, r.z > 0.f ? r.z : 0.f);
+}
+
+// ---- ray / quad -----------------------------------------------------------------------------------------
+__device__ __forceinline__ float triple(F3 d, F3 x, F3 y) {
+    return d.x * (x.y * y.z - x.z * y.y) + d.y * (x.z * y.x - x.x * y.z) + d.z * (x.x * y.y - x.y * y.x);
+}
+__device__ __forceinline__ bool same_sign(float a, float b, float c) {
+    return (a >= 0.f && b >= 0.f && c >= 0.f) || (a <= 0.f && b <= 0.f && c <= 0.f);
+}
+// Quad = triangles ABC and BCD.  Signed-volume edge tests in origin-relative coordinates, then
+// t = n.(v1-o) / n.d on the plane of the triangle that was hit.
+__device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 B, F3 C, F3 Dv, float &t, uint32_t &tri) {
+    F3 a = A - o, b = B - o, c = C - o, e = Dv - o;
+    float u0 = triple(d, b, c);
+    float u1 = triple(d, c, a);
+    float u2 = triple(d, a, b);
+    bool in0 = same_sign(u0, u1, u2);
+    float w0 = triple(d, c, e);
+    float w1 = triple(d, e, b);
+    bool in1 = same_sign(w0, w1, u0);
+    if (!(in0 || in1)) return false;
+    F3 n0 = cross(B - A, C - A);
+    F3 n1 = cross(C - B, Dv - B);
+    F3 n = in0 ? n0 : n1;
+    F3 k = in0 ? a : b;
+    tri = in0 ? 0u : 1u;
+    float p = dot(n, k);
+    float q = dot(n, d);
+    t = p / q;
+    return (t > 0.0f) && (t < kInfDepth);
+}
+
+// ---- wave-uniform fetches ---------------------------------------------------------------------------------
+typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
+template <int N>
+__device__ __forceinline__ void load_uniform(const void *p, uint32_t (&out)[N]) {
+    const_u32_ptr c = (const_u32_ptr)(uintptr_t)p;
+#pragma unroll
+    for (int k = 0; k < N; ++k) out[k] = c[k];
+}
+
+struct RaySlab {   // per-lane precomputation for the conservative slab test
+    float ix, iy, iz;     // 1/d, with tiny components pushed away from zero
+    float nx, ny, nz;     // -o * (1/d)
+    float wx, wy, wz;     // interval widening per axis
+};
+
+__device__ __forceinline__ float safe_inv(float d) {
+    float a = __builtin_fabsf(d);
+    float v = (a < 1e-20f) ? __builtin_copysignf(1e-20f, d) : d;   // NaN passes through
+    return 1.0f / v;
+}
+
+__device__ __forceinline__ RaySlab make_slab(F3 o, F3 d, float max_abs) {
+    RaySlab s;
+    s.ix = safe_inv(d.x);
+    s.iy = safe_inv(d.y);
+    s.iz = safe_inv(d.z);
+    s.nx = -o.x * s.ix;
+    s.ny = -o.y * s.iy;
+    s.nz = -o.z * s.iz;
+    // The quad test works in origin-relative fp32 coordinates, so it can accept a ray that passes
+    // a few ulps of (|o| + |vertex|) outside the quad; boxes are widened by well above that.
+    float oa = __builtin_fmaxf(__builtin_fabsf(o.x), __builtin_fmaxf(__builtin_fabsf(o.y), __builtin_fabsf(o.z)));
+    float pad = 4e-6f * (oa + max_abs);
+    s.wx = pad * __builtin_fabsf(s.ix);
+    s.wy = pad * __builtin_fabsf(s.iy);
+    s.wz = pad * __builtin_fabsf(s.iz);
+    return s;
+}
+
+// Entry distance of the ray into the widened box; the box is hit iff the result <= tmax (and tmax >= 0).
+__device__ __forceinline__ bool slab_hit(const RaySlab &s, const uint32_t *box /* lo[3],hi[3] */, float tmax, float &tn) {
+    float lx = __uint_as_float(box[0]), ly = __uint_as_float(box[1]), lz = __uint_as_float(box[2]);
+    float hx = __uint_as_float(box[3]), hy = __uint_as_float(box[4]), hz = __uint_as_float(box[5]);
+    float ax = __builtin_fmaf(lx, s.ix, s.nx), bx = __builtin_fmaf(hx, s.ix, s.nx);
+    float ay = __builtin_fmaf(ly, s.iy, s.ny), by = __builtin_fmaf(hy, s.iy, s.ny);
+    float az = __builtin_fmaf(lz, s.iz, s.nz), bz = __builtin_fmaf(hz, s.iz, s.nz);
+    float n0 = __builtin_fminf(ax, bx) - s.wx, f0 = __builtin_fmaxf(ax, bx) + s.wx;
+    float n1 = __builtin_fminf(ay, by) - s.wy, f1 = __builtin_fmaxf(ay, by) + s.wy;
+    float n2 = __builtin_fminf(az, bz) - s.wz, f2 = __builtin_fmaxf(az, bz) + s.wz;
+    tn = __builtin_fmaxf(__builtin_fmaxf(n0, n1), __builtin_fmaxf(n2, 0.0f));
+    float tf = __builtin_fminf(__builtin_fminf(f0, f1), __builtin_fminf(f2, tmax));
+    return tn <= tf;
+}
+
+// The (t, idx) pairs of the 16 nearest hits, ascending; ties in t resolved by ascending idx so that
+// the content does not depend on the order in which the BVH delivers candidates.
+struct KBuf {
+    float t[kChunk];
+    uint32_t i[kChunk];
+};
+
+__device__ __forceinline__ void kbuf_reset(KBuf &b) {
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) {
+        b.t[k] = kInfDepth;
+        b.i[k] = 0u;
+    }
+}
+
+__device__ __forceinline__ void kbuf_insert(KBuf &b, float t, uint32_t idx, bool on) {
+    float ct = t;
+    uint32_t ci = idx;
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) {
+        bool sw = on && ((ct < b.t[k]) || (ct == b.t[k] && ci < b.i[k]));
+        float tt = b.t[k];
+        uint32_t ti = b.i[k];
+        b.t[k] = sw ? ct : tt;
+        b.i[k] = sw ? ci : ti;
+        ct = sw ? tt : ct;
+        ci = sw ? ti : ci;
+    }
+}
+
+// One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
+// to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow.
+__device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
+                                           uint32_t &cnt) {
+    if (__ballot(active) == 0ull) return;
+    const RaySlab slab = make_slab(o, d, max_abs);
+    const uint32_t lane = __lane_id();
+    uint32_t stack = 0u;  // entry k lives in lane k; the tree is at most 62 levels deep (30-bit keys + index bits)
+    int sp = 0;
+    uint32_t ref = acc.root;
+    for (;;) {
+        if (ref & DST_LEAF_BIT) {
+            uint32_t L[13];
+            load_uniform<13>(&acc.leaves[ref & ~DST_LEAF_BIT], L);
+            F3 A = f3(__uint_as_float(L[0]), __uint_as_float(L[1]), __uint_as_float(L[2]));
+            F3 B = f3(__uint_as_float(L[3]), __uint_as_float(L[4]), __uint_as_float(L[5]));
+            F3 C = f3(__uint_as_float(L[6]), __uint_as_float(L[7]), __uint_as_float(L[8]));
+            F3 Dv = f3(__uint_as_float(L[9]), __uint_as_float(L[10]), __uint_as_float(L[11]));
+            float t = 0.f;
+            uint32_t tri = 0u;
+            bool hit = active && ray_quad(o, d, A, B, C, Dv, t, tri);
+            uint32_t idx = 2u * L[12] + tri;
+            bool adm = hit && ((t < buf.t[kChunk - 1]) || (t == buf.t[kChunk - 1] && idx < buf.i[kChunk - 1]));
+            if (__ballot(adm) != 0ull) {
+                cnt += adm ? 1u : 0u;
+                kbuf_insert(buf, t, idx, adm);
+            }
+            if (sp == 0) break;
+            --sp;
+            ref = __builtin_amdgcn_readlane(stack, sp);
+        } else {
+            uint32_t Nd[14];
+            load_uniform<14>(&acc.nodes[ref], Nd);
+            const float tmax = active ? buf.t[kChunk - 1] : -1.0f;
+            float tn0, tn1;
+            bool h0 = slab_hit(slab, &Nd[0], tmax, tn0);
+            bool h1 = slab_hit(slab, &Nd[6], tmax, tn1);
+            const uint64_t b0 = __ballot(h0), b1 = __ballot(h1);
+            if ((b0 | b1) == 0ull) {
+                if (sp == 0) break;
+                --sp;
+                ref = __builtin_amdgcn_readlane(stack, sp);
+            } else if (b0 != 0ull && b1 != 0ull) {
+                // both wanted: the side most lanes enter first goes first, the other is deferred
+                int v1 = __popcll(__ballot(h1 && (!h0 || tn1 < tn0)));
+                int v0 = __popcll(__ballot(h0 && (!h1 || tn0 <= tn1)));
+                uint32_t near = (v1 > v0) ? Nd[13] : Nd[12];
+                uint32_t far = (v1 > v0) ? Nd[12] : Nd[13];
+                stack = (lane == (uint32_t)sp) ? far : stack;  // entry sp lives in lane sp
+                ++sp;
+                ref = near;
+            } else {
+                ref = (b0 != 0ull) ? Nd[12] : Nd[13];
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v); }
+
+template <int AUXM>
+struct BounceIn {  // backward: saved results of the bounce and the gradients flowing into them
+    float rgb[3], dpt, acc, nrm[3], aux[AUXM];
+    float g_rgb[3], g_dpt, g_acc, g_nrm[3], g_aux[AUXM];
+};
+
+template <int AUXM>
+struct BounceAcc {
+    float C[3], D, N[3], O[AUXM], T;
+};
+
+// Gradient of one composited hit (reference backward.cu:528-640 and 201-287, 68-166).
+// Pure gradient algebra: nothing here feeds a decision, so contraction is allowed.
+template <int AUXM>
+__device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<AUXM> &in, const BounceAcc<AUXM> &run,
+                                             int g, uint32_t pidx, float Tp, float alpha, float G, float w, float dpt,
+                                             F3 xyz, const F3 (&R)[3], float u, float v, float sx, float sy, F3 mean,
+                                             float q0, float q1, float q2, float q3, float opac, float nsign,
+                                             F3 normal, const float (&col)[3], const bool (&neg)[3], F3 ro, F3 rd,
+                                             const float *__restrict__ sh, F3 &g_ro, F3 &g_rd) {
+#pragma clang fp contract(fast)
+    const float num = 1.0f - alpha;
+    const float T_final = 1.0f - in.acc;
+    float g_alpha = 0.f;
+    float g_col[3];
+#pragma unroll
+    for (int ch = 0; ch < 3; ++ch) {
+        g_col[ch] = in.g_rgb[ch] * w;
+        aadd(p.dL_dcolors + 3 * (size_t)g + ch, g_col[ch]);
+        g_alpha += in.g_rgb[ch] * (Tp * col[ch] - (in.rgb[ch] - run.C[ch]) / num);
+        g_alpha += in.g_rgb[ch] * p.background[ch] * (-T_final / num);
+    }
+    if (p.others_precomp != nullptr) {
+#pragma unroll
+        for (int ch = 0; ch < AUXM; ++ch) {
+            if (ch < p.aux) {
+                float o = p.others_precomp[(size_t)p.aux * g + ch];
+                aadd(p.dL_dothers + (size_t)p.aux * g + ch, in.g_aux[ch] * w);
+                g_alpha += in.g_aux[ch] * (Tp * o - (in.aux[ch] - run.O[ch]) / num);
+            }
+        }
+    }
+    const float g_D = in.g_dpt * w;
+    g_alpha += in.g_dpt * (Tp * dpt - (in.dpt - run.D) / num);
+    const F3 g_N = f3(in.g_nrm[0] * w, in.g_nrm[1] * w, in.g_nrm[2] * w);
+    g_alpha += in.g_nrm[0] * (Tp * normal.x - (in.nrm[0] - run.N[0]) / num) +
+               in.g_nrm[1] * (Tp * normal.y - (in.nrm[1] - run.N[1]) / num) +
+               in.g_nrm[2] * (Tp * normal.z - (in.nrm[2] - run.N[2]) / num);
+    g_alpha += in.g_acc * (Tp - in.acc / num);   // the reference never accumulates W (backward.cu:568)
+    const float g_G = g_alpha * opac;
+    const float pc = (opac * G) > 0.99f ? 0.0f : 1.0f;
+    aadd(p.dL_dopacities + g, g_alpha * G * pc);
+
+    // triangle that was hit, with its corner coordinates in splat units (backward.cu:583-602)
+    const float *V = p.vertices + (size_t)g * 12;
+    F3 v1, v2, v3, h1, h2, h3;
+    if ((pidx & 1u) == 0u) {
+        v1 = ld3(V); v2 = ld3(V + 3); v3 = ld3(V + 6);
+        h1 = f3(-3.f, 3.f, 3.f); h2 = f3(-3.f, -3.f, 3.f); h3 = f3(3.f, 3.f, 3.f);
+    } else {
+        v1 = ld3(V + 3); v2 = ld3(V + 6); v3 = ld3(V + 9);
+        h1 = f3(-3.f, -3.f, 3.f); h2 = f3(3.f, 3.f, 3.f); h3 = f3(3.f, -3.f, 3.f);
+    }
+    const float k = g_G * pc;
+    const float gu = k * -G * u, gv = k * -G * v;
+    F3 gR[3];
+    const F3 rel = xyz - mean;
+    gR[0] = gu * rel / sx;
+    gR[1] = gv * rel / sy;
+    gR[2] = g_N * nsign;
+    float g_sx = k * (G * u * u / sx), g_sy = k * (G * v * v / sy);
+    F3 g_mean = k * (G * (R[0] * u / sx + R[1] * v / sy));
+    const F3 g_xyz = (gu / sx) * R[0] + (gv / sy) * R[1];
+    const float g_d = g_D + dot(g_xyz, rd);
+    const F3 n = cross(v2 - v1, v3 - v1);
+    const F3 c = v1 - ro;
+    const float pp = dot(n, c), q = dot(n, rd);
+    const F3 g_n = (c - (pp / q) * rd) / q;
+    const F3 g_v1 = g_d * cross(v2 - v3, g_n) + g_d * n / q;
+    const F3 g_v2 = g_d * cross(v3 - v1, g_n);
+    const F3 g_v3 = g_d * cross(v1 - v2, g_n);
+    g_ro = g_ro + (g_xyz + (g_d * -n) / q);
+    g_rd = g_rd + (g_xyz * dpt + ((g_d * -pp) / (q * q)) * n);
+    const F3 su = h1.x * g_v1 + h2.x * g_v2 + h3.x * g_v3;
+    const F3 sv = h1.y * g_v1 + h2.y * g_v2 + h3.y * g_v3;
+    gR[0] = gR[0] + sx * su;
+    gR[1] = gR[1] + sy * sv;
+    g_sx += dot(R[0], su);
+    g_sy += dot(R[1], sv);
+    g_mean = g_mean + (g_v1 + g_v2 + g_v3);
+    // rotation: vjp of quat_rows without the normalisation Jacobian (auxiliary.h:433-477)
+    {
+        float s = 1.0f / __builtin_sqrtf(q3 * q3 + q0 * q0 + q1 * q1 + q2 * q2);
+        float w_ = q0 * s, x = q1 * s, y = q2 * s, z = q3 * s;
+        float r0 = 2.f * (x * (gR[1].z - gR[2].y) + y * (gR[2].x - gR[0].z) + z * (gR[0].y - gR[1].x));
+        float r1 = 2.f * (-2.f * x * (gR[1].y + gR[2].z) + y * (gR[0].y + gR[1].x) + z * (gR[0].z + gR[2].x) +
+                          w_ * (gR[1].z - gR[2].y));
+        float r2 = 2.f * (x * (gR[0].y + gR[1].x) - 2.f * y * (gR[0].x + gR[2].z) + z * (gR[1].z + gR[2].y) +
+                          w_ * (gR[2].x - gR[0].z));
+        float r3 = 2.f * (x * (gR[0].z + gR[2].x) + y * (gR[1].z + gR[2].y) - 2.f * z * (gR[0].x + gR[1].y) +
+                          w_ * (gR[0].y - gR[1].x));
+        float *dr = p.dL_drotations + 4 * (size_t)g;
+        aadd(dr + 0, r0); aadd(dr + 1, r1); aadd(dr + 2, r2); aadd(dr + 3, r3);
+    }
+    aadd(p.dL_dscales + 2 * (size_t)g + 0, g_sx);
+    aadd(p.dL_dscales + 2 * (size_t)g + 1, g_sy);
+    float *dm = p.dL_dmeans3D + 3 * (size_t)g, *dg = p.dL_dgrads3D + 3 * (size_t)g;
+    aadd(dm + 0, g_mean.x); aadd(dm + 1, g_mean.y); aadd(dm + 2, g_mean.z);
+    const float hd = 0.5f * dpt;
+    aadd(dg + 0, g_mean.x * hd); aadd(dg + 1, g_mean.y * hd); aadd(dg + 2, g_mean.z * hd);
+
+    if (p.colors_precomp == nullptr) {
+        // SH backward (backward.cu:68-166); the direction gradient REPLACES the ray's (backward.cu:165)
+        const int deg = p.D;
+        F3 gc = f3(neg[0] ? 0.f : g_col[0], neg[1] ? 0.f : g_col[1], neg[2] ? 0.f : g_col[2]);
+        float *ds = p.dL_dshs + (size_t)g * p.M * 3;
+        auto put = [&](int j, float basis) {
+            aadd(ds + 3 * j + 0, basis * gc.x);
+            aadd(ds + 3 * j + 1, basis * gc.y);
+            aadd(ds + 3 * j + 2, basis * gc.z);
+        };
+        auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
+        F3 ddx = f3(0, 0, 0), ddy = f3(0, 0, 0), ddz = f3(0, 0, 0);
+        const float x = rd.x, y = rd.y, z = rd.z;
+        put(0, SH0);
+        if (deg > 0) {
+            put(1, -SH1 * y);
+            put(2, SH1 * z);
+            put(3, -SH1 * x);
+            ddx = -SH1 * S(3);
+            ddy = -SH1 * S(1);
+            ddz = SH1 * S(2);
+            if (deg > 1) {
+                const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+                put(4, SH2[0] * xy);
+                put(5, SH2[1] * yz);
+                put(6, SH2[2] * (2.f * zz - xx - yy));
+                put(7, SH2[3] * xz);
+                put(8, SH2[4] * (xx - yy));
+                ddx = ddx + SH2[0] * y * S(4) + SH2[2] * 2.f * -x * S(6) + SH2[3] * z * S(7) + SH2[4] * 2.f * x * S(8);
+                ddy = ddy + SH2[0] * x * S(4) + SH2[1] * z * S(5) + SH2[2] * 2.f * -y * S(6) + SH2[4] * 2.f * -y * S(8);
+                ddz = ddz + SH2[1] * y * S(5) + SH2[2] * 4.f * z * S(6) + SH2[3] * x * S(7);
+                if (deg > 2) {
+                    put(9, SH3[0] * y * (3.f * xx - yy));
+                    put(10, SH3[1] * xy * z);
+                    put(11, SH3[2] * y * (4.f * zz - xx - yy));
+                    put(12, SH3[3] * z * (2.f * zz - 3.f * xx - 3.f * yy));
+                    put(13, SH3[4] * x * (4.f * zz - xx - yy));
+                    put(14, SH3[5] * z * (xx - yy));
+                    put(15, SH3[6] * x * (xx - 3.f * yy));
+                    ddx = ddx + (SH3[0] * 6.f * xy) * S(9) + (SH3[1] * yz) * S(10) + (SH3[2] * -2.f * xy) * S(11) +
+                          (SH3[3] * -6.f * xz) * S(12) + (SH3[4] * (-3.f * xx + 4.f * zz - yy)) * S(13) +
+                          (SH3[5] * 2.f * xz) * S(14) + (SH3[6] * 3.f * (xx - yy)) * S(15);
+                    ddy = ddy + (SH3[0] * 3.f * (xx - yy)) * S(9) + (SH3[1] * xz) * S(10) +
+                          (SH3[2] * (-3.f * yy + 4.f * zz - xx)) * S(11) + (SH3[3] * -6.f * yz) * S(12) +
+                          (SH3[4] * -2.f * xy) * S(13) + (SH3[5] * -2.f * yz) * S(14) + (SH3[6] * -6.f * xy) * S(15);
+                    ddz = ddz + (SH3[1] * xy) * S(10) + (SH3[2] * 8.f * yz) * S(11) +
+                          (SH3[3] * 3.f * (2.f * zz - xx - yy)) * S(12) + (SH3[4] * 8.f * xz) * S(13) +
+                          (SH3[5] * (xx - yy)) * S(14);
+                }
+            }
+        }
+        g_rd = f3(dot(ddx, gc), dot(ddy, gc), dot(ddz, gc));
+    }
+}
+
+// One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
+// and for BWD the per-hit gradients of the re-trace (reference backward.cu:332-655).
+template <bool BWD, int AUXM>
+__device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
+                                            F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
+                                            const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
+                                            uint32_t &n_con) {
+    run.C[0] = run.C[1] = run.C[2] = 0.f;
+    run.D = 0.f;
+    run.N[0] = run.N[1] = run.N[2] = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < AUXM; ++ch) run.O[ch] = 0.f;
+    float pay_dpt = 0.f, dpt = 0.f, Tp = 1.f, Tn = 1.f;
+    int last_g = -1, contrib = 0;
+    F3 ot = ro;
+    bool live = lane_on;
+    KBuf buf;
+    while (__ballot(live) != 0ull) {
+        kbuf_reset(buf);
+        uint32_t cnt = 0;
+        packet_knn(acc, max_abs, ot, rd, live, buf, cnt);
+        int here = 0;
+        bool stop = false;
+        for (int it = 0; it < kChunk; ++it) {
+            const bool on = live && !stop && (uint32_t)it < cnt;
+            if (__ballot(on) == 0ull) break;
+            // pop the front entry; the rest moves up (consumed slots need no reset: the buffer is
+            // rebuilt from scratch for the next chunk)
+            const float e_t = buf.t[0];
+            const uint32_t e_i = buf.i[0];
+#pragma unroll
+            for (int k = 0; k < kChunk - 1; ++k) {
+                buf.t[k] = buf.t[k + 1];
+                buf.i[k] = buf.i[k + 1];
+            }
+            if (!on) continue;
+            const int g = (int)(e_i >> 1);
+            if (g == last_g) continue;
+            dpt = e_t + pay_dpt;
+            const F3 xyz = f3(ro.x + dpt * rd.x, ro.y + dpt * rd.y, ro.z + dpt * rd.z);
+            const F3 mean = ld3(p.means3D + 3 * (size_t)g);
+            const float sx = p.scales[2 * (size_t)g], sy = p.scales[2 * (size_t)g + 1];
+            const float *qp = p.rotations + 4 * (size_t)g;
+            const float q0 = qp[0], q1 = qp[1], q2 = qp[2], q3 = qp[3];
+            F3 R[3];
+            quat_rows(q0, q1, q2, q3, R);
+            const float Tx = dot(R[0], mean), Ty = dot(R[1], mean);
+            const float ux = R[0].x * xyz.x + R[0].y * xyz.y + R[0].z * xyz.z + (-Tx);
+            const float uy = R[1].x * xyz.x + R[1].y * xyz.y + R[1].z * xyz.z + (-Ty);
+            const float u = ux / sx, v = uy / sy;
+            const float rho = u * u + v * v;
+            n_proc++;
+            F3 normal = R[2];
+            const float cosv = -(rd.x * normal.x + rd.y * normal.y + rd.z * normal.z);
+            if (cosv == 0.f) continue;
+            const float nsign = cosv > 0.f ? 1.0f : -1.0f;
+            normal = cosv > 0.f ? normal : -normal;
+            if (dpt < min_depth) continue;
+            const float power = -0.5f * rho;
+            if (power > 0.0f) continue;
+            const float opac = p.opacities[g];
+            const float G = exp_det(power);
+            float alpha = opac * G;
+            alpha = (alpha < 0.99f) ? alpha : 0.99f;
+            if (alpha < 1.0f / 255.0f) continue;
+            Tn = Tp * (1 - alpha);
+            if (Tn < kTmin) { stop = true; continue; }
+            contrib++;
+            if (contrib > kMaxContrib) { stop = true; continue; }
+            last_g = g;
+            const float w = alpha * Tp;
+            float col[3];
+            bool neg[3] = {false, false, false};
+            const float *sh = nullptr;
+            if (p.colors_precomp == nullptr) {
+                sh = p.shs + (size_t)g * p.M * 3;
+                F3 c = sh_color(p.D, sh, rd, neg);
+                col[0] = c.x; col[1] = c.y; col[2] = c.z;
+            } else {
+                col[0] = p.colors_precomp[3 * (size_t)g];
+                col[1] = p.colors_precomp[3 * (size_t)g + 1];
+                col[2] = p.colors_precomp[3 * (size_t)g + 2];
+            }
+            run.C[0] += w * col[0];
+            run.C[1] += w * col[1];
+            run.C[2] += w * col[2];
+            if (p.others_precomp != nullptr) {
+#pragma unroll
+                for (int ch = 0; ch < AUXM; ++ch)
+                    if (ch < p.aux) run.O[ch] += w * p.others_precomp[(size_t)p.aux * g + ch];
+            }
+            run.D += w * dpt;
+            run.N[0] += w * normal.x;
+            run.N[1] += w * normal.y;
+            run.N[2] += w * normal.z;
+            n_con++;
+            here++;
+            if (BWD) {
+                hit_backward<AUXM>(p, in, run, g, e_i, Tp, alpha, G, w, dpt, xyz, R, u, v, sx, sy, mean, q0, q1, q2, q3,
+                                   opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd);
+            } else if (p.training && p.a_weights != nullptr) {
+                aadd(p.a_weights + g, w);
+            }
+            Tp = Tn;
+        }
+        if (live) {
+            bool fin = (Tn < kTmin) || (cnt < (uint32_t)kChunk) || (contrib > kMaxContrib);
+            const float next_dpt = (float)((double)dpt + kStepEps);
+            if (!(next_dpt > pay_dpt) && here == 0) fin = true;   // the reference would never leave this state
+            if (fin) {
+                live = false;
+            } else {
+                pay_dpt = next_dpt;
+                ot = f3(ro.x + pay_dpt * rd.x, ro.y + pay_dpt * rd.y, ro.z + pay_dpt * rd.z);
+            }
+        }
+    }
+    run.T = Tp;
+}
+
+__device__ __forceinline__ F3 dnormvdv(F3 v, F3 dv) {
+    float sum2 = v.x * v.x + v.y * v.y + v.z * v.z;
+    float inv = 1.0f / __builtin_sqrtf(sum2 * sum2 * sum2);
+    return f3(((+sum2 - v.x * v.x) * dv.x - v.y * v.x * dv.y - v.z * v.x * dv.z) * inv,
+              (-v.x * v.y * dv.x + (sum2 - v.y * v.y) * dv.y - v.z * v.y * dv.z) * inv,
+              (-v.x * v.z * dv.x - v.y * v.z * dv.y + (sum2 - v.z * v.z) * dv.z) * inv);
+}
+__device__ __forceinline__ F3 ddotndndn(F3 n, F3 d, F3 g) {
+    float nd = dot(n, d);
+    return f3(g.x * (nd + d.x * n.x) + g.y * d.x * n.y + g.z * d.x * n.z,
+              g.x * d.y * n.x + g.y * (nd + d.y * n.y) + g.z * d.y * n.z,
+              g.x * d.z * n.x + g.y * d.z * n.y + g.z * (nd + d.z * n.z));
+}
+__device__ __forceinline__ F3 ddotndndd(F3 n, F3 g) {
+    return f3(g.x * n.x * n.x + g.y * n.x * n.y + g.z * n.x * n.z, g.x * n.y * n.x + g.y * n.y * n.y + g.z * n.y * n.z,
+              g.x * n.z * n.x + g.y * n.z * n.y + g.z * n.z * n.z);
+}
+
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+template <bool BWD, int AUXM>
+__global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstParams p, const DstAccelView acc,
+                                                                     int tw_log2, int th_log2, uint32_t tiles_x,
+                                                                     uint32_t n_tiles) {
+    const uint32_t tile = blockIdx.x * kWavesPerBlock + (threadIdx.x / DST_WAVE);
+    if (tile >= n_tiles) return;
+    const uint32_t lane = threadIdx.x % DST_WAVE;
+    const uint32_t ty = tile / tiles_x, tx = tile % tiles_x;
+    const uint32_t py = (ty << th_log2) + (lane >> tw_log2);
+    const uint32_t px = (tx << tw_log2) + (lane & ((1u << tw_log2) - 1u));
+    const bool inside = py < (uint32_t)p.H && px < (uint32_t)p.W;
+    const size_t r = inside ? ((size_t)py * p.W + px) : 0;
+    const float max_abs = __uint_as_float(acc.bounds->max_abs);
+    const int MID = 14 + p.aux, AUXO = 11, RGBO = 11 + p.aux;
+    const int slots = p.mtd_alloc + 1, mtd = p.max_trace_depth;
+    float *mid = p.mid_val + (size_t)slots * MID * r;
+    const F3 ray_o = ld3(p.ray_o + 3 * r), ray_d = ld3(p.ray_d + 3 * r);
+    uint32_t n_proc = 0, n_con = 0;
+    BounceAcc<AUXM> run;
+    BounceIn<AUXM> in;
+    F3 g_ro = f3(0, 0, 0), g_rd = f3(0, 0, 0);
+
+    if (!BWD) {
+        // reference forward.cu:318-424
+        float out_rgb[3] = {0.f, 0.f, 0.f};
+        F3 ot = ray_o, dt = ray_d;
+        float s_prod = 1.0f;
+        bool on = inside;
+        for (int i = 0; i <= mtd; ++i) {
+            const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
+            walk_bounce<false, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con);
+            if (on) {
+                run.C[0] += run.T * p.background[0];
+                run.C[1] += run.T * p.background[1];
+                run.C[2] += run.T * p.background[2];
+                const float A = 1 - run.T;
+                const F3 E = f3(ot.x + run.D * dt.x, ot.y + run.D * dt.y, ot.z + run.D * dt.z);
+                if (i == 0) {
+                    p.out_dpt[r] = run.D;
+                    p.out_acc[r] = A;
+                    p.out_norm[3 * r + 0] = run.N[0];
+                    p.out_norm[3 * r + 1] = run.N[1];
+                    p.out_norm[3 * r + 2] = run.N[2];
+                    p.out_dist[3 * r + 0] = 0.f;
+                    p.out_dist[3 * r + 1] = 0.f;
+                    p.out_dist[3 * r + 2] = 0.f;
+#pragma unroll
+                    for (int ch = 0; ch < AUXM; ++ch)
+                        if (ch < p.aux) p.out_aux[(size_t)p.aux * r + ch] = run.O[ch];
+                }
+                const float f_this = (i == mtd) ? 1.0f : 1 - run.O[0];
+                out_rgb[0] += run.C[0] * f_this * s_prod;
+                out_rgb[1] += run.C[1] * f_this * s_prod;
+                out_rgb[2] += run.C[2] * f_this * s_prod;
+                s_prod *= run.O[0];
+                float *m = mid + (size_t)i * MID;
+                m[0] = ot.x; m[1] = ot.y; m[2] = ot.z;
+                m[3] = dt.x; m[4] = dt.y; m[5] = dt.z;
+                m[6] = run.D;
+                m[7] = A;
+                m[8] = run.N[0]; m[9] = run.N[1]; m[10] = run.N[2];
+#pragma unroll
+                for (int ch = 0; ch < AUXM; ++ch)
+                    if (ch < p.aux) m[AUXO + ch] = run.O[ch];
+                m[RGBO + 0] = run.C[0];
+                m[RGBO + 1] = run.C[1];
+                m[RGBO + 2] = run.C[2];
+                const F3 N = f3(run.N[0], run.N[1], run.N[2]);
+                const float nl = length(N);
+                if (nl == 0.0f || run.O[0] <= p.specular_threshold) {
+                    on = false;
+                    // slots of the bounces never traced read as zeros
+                    for (int k = (i + 1) * MID; k < slots * MID; ++k) mid[k] = 0.f;
+                } else {
+                    const F3 n = N / nl;
+                    dt = dt - 2 * dot(n, dt) * n;
+                    ot = E + kStartOffset * dt;
+                }
+            }
+        }
+        if (inside) {
+            if (on)
+                for (int k = (mtd + 1) * MID; k < slots * MID; ++k) mid[k] = 0.f;
+            p.out_rgb[3 * r + 0] = out_rgb[0];
+            p.out_rgb[3 * r + 1] = out_rgb[1];
+            p.out_rgb[3 * r + 2] = out_rgb[2];
+        }
+        if (p.counters != nullptr) {
+            uint32_t a = wave_sum(n_proc), b = wave_sum(n_con);
+            if (lane == 0) {
+                atomicAdd(p.counters + 0, (unsigned long long)a);
+                atomicAdd(p.counters + 1, (unsigned long long)b);
+            }
+        }
+    } else {
+        // reference backward.cu:658-853
+        float C_prev[3], c_prev[3] = {0.f, 0.f, 0.f}, g_out_rgb[3];
+        for (int ch = 0; ch < 3; ++ch) {
+            C_prev[ch] = p.out_rgb[3 * r + ch];
+            g_out_rgb[ch] = p.dL_drgb[3 * r + ch];
+        }
+        float s_prod = 1.0f;
+        for (int i = 0; i < mtd; ++i) {
+            for (int ch = 0; ch < 3; ++ch) {
+                float c_curr = mid[ch + RGBO + i * MID];
+                C_prev[ch] = C_prev[ch] + s_prod * (c_prev[ch] - c_curr);
+                c_prev[ch] = c_curr;
+            }
+            s_prod *= mid[AUXO + i * MID];
+        }
+        for (int i = mtd; i >= 0; --i) {
+            const float *m = mid + (size_t)i * MID;
+            const F3 ot = ld3(m), dt = ld3(m + 3);
+            const float s_prev = (i > 0) ? mid[AUXO + (i - 1) * MID] : 1.0f;
+            const bool on = inside && !(length(dt) == 0.0f || s_prev <= p.specular_threshold);
+            if (on) {
+                for (int ch = 0; ch < 3; ++ch) in.rgb[ch] = m[RGBO + ch];
+                in.dpt = m[6];
+                in.acc = m[7];
+                in.nrm[0] = m[8]; in.nrm[1] = m[9]; in.nrm[2] = m[10];
+#pragma unroll
+                for (int ch = 0; ch < AUXM; ++ch) {
+                    in.aux[ch] = (ch < p.aux) ? m[AUXO + ch] : 0.f;
+                    in.g_aux[ch] = 0.f;
+                }
+                in.g_dpt = 0.f;
+                in.g_acc = 0.f;
+                in.g_nrm[0] = in.g_nrm[1] = in.g_nrm[2] = 0.f;
+                const float f_this = (i == mtd) ? 1.0f : 1 - in.aux[0];
+                for (int ch = 0; ch < 3; ++ch) in.g_rgb[ch] = g_out_rgb[ch] * f_this * s_prod;
+                s_prod /= s_prev;
+                if (i != mtd) {
+                    for (int ch = 0; ch < 3; ++ch) {
+                        in.g_aux[0] += g_out_rgb[ch] * (C_prev[ch] / in.aux[0]);
+                        c_prev[ch] = (i > 0) ? mid[ch + RGBO + (i - 1) * MID] : 0.0f;
+                        C_prev[ch] = C_prev[ch] - s_prod * (c_prev[ch] - in.rgb[ch]);
+                    }
+                    const F3 nrm = f3(in.nrm[0], in.nrm[1], in.nrm[2]);
+                    const float nl = length(nrm);
+                    if (nl != 0.f) {
+                        g_rd = g_rd + g_ro * (float)kStepEps;
+                        const F3 n = nrm / nl;
+                        in.g_dpt += g_ro.x * dt.x + g_ro.y * dt.y + g_ro.z * dt.z;
+                        const F3 gn = dnormvdv(nrm, ddotndndn(n, dt, g_rd * -2.0f));
+                        in.g_nrm[0] += gn.x;
+                        in.g_nrm[1] += gn.y;
+                        in.g_nrm[2] += gn.z;
+                        g_rd = g_ro * in.dpt + g_rd + ddotndndd(n, g_rd * -2.0f);
+                    }
+                }
+                if (i == 0) {
+                    in.g_dpt += p.dL_ddpt[r];
+                    in.g_acc += p.dL_dacc[r];
+                    in.g_nrm[0] += p.dL_dnorm[3 * r + 0];
+                    in.g_nrm[1] += p.dL_dnorm[3 * r + 1];
+                    in.g_nrm[2] += p.dL_dnorm[3 * r + 2];
+#pragma unroll
+                    for (int ch = 0; ch < AUXM; ++ch)
+                        if (ch < p.aux) in.g_aux[ch] += p.dL_daux[(size_t)p.aux * r + ch];
+                }
+            }
+            const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
+            walk_bounce<true, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con);
+        }
+        if (inside) {
+            p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
+            p.dL_dray_d[3 * r + 0] = g_rd.x; p.dL_dray_d[3 * r + 1] = g_rd.y; p.dL_dray_d[3 * r + 2] = g_rd.z;
+        }
+    }
+}
+
+template <bool BWD>
+void launch(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2, uint32_t tiles_x, uint32_t n_tiles,
+            hipStream_t stream) {
+    dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock), block(kWavesPerBlock * DST_WAVE);
+    if (p.aux <= 2)
+        hipLaunchKernelGGL((k_trace<BWD, 2>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, n_tiles);
+    else if (p.aux <= 4)
+        hipLaunchKernelGGL((k_trace<BWD, 4>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, n_tiles);
+    else
+        hipLaunchKernelGGL((k_trace<BWD, 8>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, n_tiles);
+}
+
+}  // namespace
+
+int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream) {
+    if (p.H <= 0 || p.W <= 0) return DST_OK;  // empty ray grid: nothing to do
+    // 8x8 pixel tiles per wave; thin grids (H < 8, e.g. (1,N,3) ray lists) get wider, flatter tiles
+    int th_log2 = 3;
+    while (th_log2 > 0 && (1 << th_log2) > p.H) --th_log2;
+    const int tw_log2 = 6 - th_log2;
+    const uint32_t tiles_x = ((uint32_t)p.W + (1u << tw_log2) - 1) >> tw_log2;
+    const uint32_t tiles_y = ((uint32_t)p.H + (1u << th_log2) - 1) >> th_log2;
+    const uint64_t n_tiles64 = (uint64_t)tiles_x * tiles_y;
+    if (n_tiles64 > 0x7FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
+    DstAccelView acc;
+    acc.nodes = ctx->nodes;
+    acc.leaves = ctx->leaves;
+    acc.bounds = ctx->bounds;
+    acc.n_leaves = ctx->n_leaves;
+    acc.root = (ctx->n_leaves == 1) ? (DST_LEAF_BIT | 0u) : 0u;
+    if (backward)
+        launch<true>(p, acc, tw_log2, th_log2, tiles_x, (uint32_t)n_tiles64, stream);
+    else
+        launch<false>(p, acc, tw_log2, th_log2, tiles_x, (uint32_t)n_tiles64, stream);
+    DST_HIP(ctx, hipGetLastError());
+    return DST_OK;
+}

@@ -1,0 +1,248 @@
+"""ctypes binding of libdst.so, shaped like the compiled `_C` module of the reference package
+(reference ext.cpp:7-12): `OptiXStateWrapper`, `build_acceleration_structure`, `trace_surfels`,
+`trace_surfels_backward` with the same positional arguments and return tuples
+(reference trace_surfels.h:10-83).  There is no fallback: a missing library raises.
+"""
+import ctypes as C
+import os
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libdst.so")
+
+NUM_CHANNELS = 3          # reference optix_tracer/config.h:5
+DEFAULT_AUX_CHANNELS = 2  # reference optix_tracer/config.h:6
+DEFAULT_MAX_TRACE_DEPTH = 1  # reference optix_tracer/config.h:27: mid_val always holds at least two slots
+MAX_AUX_CHANNELS = 8
+MAX_TRACE_DEPTH = 3
+
+_FP = C.c_void_p
+
+
+class DstParams(C.Structure):
+    """Field-for-field mirror of `DstParams` in include/dst_api.h."""
+    _fields_ = (
+        [(n, C.c_int32) for n in ("P", "H", "W", "D", "M", "aux", "mtd_alloc", "max_trace_depth", "training",
+                                  "start_from_first")]
+        + [("specular_threshold", C.c_float), ("scale_modifier", C.c_float)]
+        + [(n, _FP) for n in ("ray_o", "ray_d", "vertices", "background", "means3D", "shs", "colors_precomp",
+                              "others_precomp", "opacities", "scales", "rotations")]
+        + [(n, _FP) for n in ("out_rgb", "out_dpt", "out_acc", "out_norm", "out_dist", "out_aux", "mid_val",
+                              "a_weights", "counters")]
+        + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
+        + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
+                              "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
+    )
+
+
+class DstAccelInfo(C.Structure):
+    _fields_ = [("n_surfels", C.c_uint32), ("n_internal", C.c_uint32), ("root", C.c_uint32),
+                ("node_bytes", C.c_uint32), ("leaf_bytes", C.c_uint32), ("scene_lo", C.c_float * 3),
+                ("scene_hi", C.c_float * 3), ("max_abs", C.c_float), ("builds", C.c_uint32), ("refits", C.c_uint32)]
+
+
+EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
+           "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params")
+
+_lib = None
+
+
+def load_library():
+    """Load libdst.so (once) and declare its prototypes.  Raises if the library is absent or stale."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("diff_surfel_tracing: %s is missing; build it with `make -C csrc` (hipcc, gfx950). "
+                          "There is no CPU or PyTorch fallback." % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    L.dst_create.restype = C.c_void_p
+    L.dst_create.argtypes = []
+    L.dst_destroy.restype = None
+    L.dst_destroy.argtypes = [C.c_void_p]
+    L.dst_build_accel.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_int, C.c_void_p]
+    L.dst_trace_forward.argtypes = [C.c_void_p, C.POINTER(DstParams), C.c_void_p]
+    L.dst_trace_backward.argtypes = [C.c_void_p, C.POINTER(DstParams), C.c_void_p]
+    L.dst_last_error.restype = C.c_char_p
+    L.dst_last_error.argtypes = [C.c_void_p]
+    L.dst_accel_info.argtypes = [C.c_void_p, C.POINTER(DstAccelInfo)]
+    L.dst_accel_download.argtypes = [C.c_void_p] * 7
+    L.dst_version.restype = C.c_char_p
+    L.dst_sizeof_params.restype = C.c_size_t
+    if L.dst_sizeof_params() != C.sizeof(DstParams):
+        raise ImportError("diff_surfel_tracing: DstParams layout mismatch between _C.py and libdst.so")
+    _lib = L
+    return L
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(ctx, rc):
+    if rc != 0:
+        msg = load_library().dst_last_error(ctx.handle)
+        raise RuntimeError((msg or b"unknown error").decode() + " (status %d)" % rc)
+
+
+def _cuda_f32(t, name):
+    """The launcher's tensor contract: CUDA, fp32, contiguous (reference trace_surfels.cpp:23-24,252-277)."""
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError("%s must be a tensor" % name)
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if t.dtype != torch.float32:
+        t = t.float()
+    return t.contiguous()
+
+
+def _ptr(t):
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+class OptiXStateWrapper:
+    """Owner of the acceleration structure; keeps the reference's class name (ext.cpp:8) so callers need not
+    change.  `pkg_dir` was where the reference looked for its PTX files and is ignored."""
+
+    def __init__(self, pkg_dir=None):
+        lib = load_library()
+        if not torch.cuda.is_available():
+            raise RuntimeError("diff_surfel_tracing needs a GPU: no HIP device is visible")
+        self.handle = lib.dst_create()
+        if not self.handle:
+            raise RuntimeError("dst_create failed: no usable HIP device")
+        self.device = torch.cuda.current_device()
+        self.num_surfels = 0
+
+    def accel_info(self):
+        info = DstAccelInfo()
+        _check(self, load_library().dst_accel_info(self.handle, C.byref(info)))
+        return info
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h and _lib is not None:
+            _lib.dst_destroy(h)
+
+
+def build_acceleration_structure(ctx, vertices, triangles, rebuild):
+    """Reference BuildAccelerationStructure (trace_surfels.cpp:36-159)."""
+    if vertices.dim() != 2 or vertices.size(1) != 3:
+        raise RuntimeError("vertices must have dimensions (num_vertices, 3)")
+    if triangles.dim() != 2 or triangles.size(1) != 3:
+        raise RuntimeError("triangles must have dimensions (num_triangles, 3)")
+    v = _cuda_f32(vertices, "vertices")
+    if not triangles.is_cuda:
+        raise RuntimeError("triangles must be a CUDA tensor")
+    f = triangles.to(torch.int32).contiguous()
+    rc = load_library().dst_build_accel(ctx.handle, v.data_ptr(), v.size(0), f.data_ptr(), f.size(0),
+                                        int(bool(rebuild)), _stream())
+    _check(ctx, rc)
+    ctx.num_surfels = f.size(0) // 2
+
+
+def _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp, others_precomp,
+                   opacities, scales, scale_modifier, rotations, max_trace_depth, specular_threshold,
+                   start_from_first):
+    if means3D.dim() != 2 or means3D.size(1) != 3:
+        raise RuntimeError("means3D must have dimensions (num_points, 3)")
+    t = {
+        "ray_o": _cuda_f32(ray_o, "ray_o"), "ray_d": _cuda_f32(ray_d, "ray_d"),
+        "vertices": _cuda_f32(vertices, "vertices"), "background": _cuda_f32(background, "background"),
+        "means3D": _cuda_f32(means3D, "means3D"), "shs": _cuda_f32(shs, "shs"),
+        "colors_precomp": _cuda_f32(colors_precomp, "colors_precomp"),
+        "others_precomp": _cuda_f32(others_precomp, "others_precomp"),
+        "opacities": _cuda_f32(opacities, "opacities"), "scales": _cuda_f32(scales, "scales"),
+        "rotations": _cuda_f32(rotations, "rotations"),
+    }
+    if t["ray_o"].dim() != 3 or t["ray_o"].size(2) != 3 or t["ray_d"].shape != t["ray_o"].shape:
+        raise RuntimeError("ray_o and ray_d must have the same dimensions (H, W, 3) or (B, P, 3)")
+    if t["scales"].numel() == 0 or t["rotations"].numel() == 0:
+        raise RuntimeError("scales and rotations are required (a precomputed 3D covariance is not consumed by "
+                           "the tracer)")
+    p = DstParams()
+    p.P, p.H, p.W = means3D.size(0), t["ray_o"].size(0), t["ray_o"].size(1)
+    p.D = int(degree)
+    p.M = t["shs"].size(1) if t["shs"].numel() != 0 else 0
+    p.aux = t["others_precomp"].size(1) if t["others_precomp"].numel() != 0 else DEFAULT_AUX_CHANNELS
+    p.max_trace_depth = int(max_trace_depth)
+    p.mtd_alloc = max(DEFAULT_MAX_TRACE_DEPTH, p.max_trace_depth)
+    p.start_from_first = int(bool(start_from_first))
+    p.specular_threshold = float(specular_threshold)
+    p.scale_modifier = float(scale_modifier)
+    for name, ten in t.items():
+        setattr(p, name, _ptr(ten))
+    return p, t
+
+
+def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, background, means3D, shs, degree,
+                  colors_precomp, others_precomp, opacities, scales, scale_modifier, rotations, transMat_precomp,
+                  viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth, specular_threshold,
+                  counters=None):
+    """Reference TraceSurfelsCUDA (trace_surfels.cpp:162-304): returns
+    (out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights or None)."""
+    p, keep = _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp,
+                             others_precomp, opacities, scales, scale_modifier, rotations, max_trace_depth,
+                             specular_threshold, start_from_first)
+    H, W, P, dev = p.H, p.W, p.P, means3D.device
+    mid_ch = (14 + p.aux) * (p.mtd_alloc + 1)
+    new = lambda *shape: torch.empty(shape, dtype=torch.float32, device=dev)  # noqa: E731 (kernel writes every element)
+    out_rgb, out_dpt, out_acc = new(H, W, NUM_CHANNELS), new(H, W, 1), new(H, W, 1)
+    out_norm, out_dist, out_aux, mid_val = new(H, W, 3), new(H, W, 3), new(H, W, p.aux), new(H, W, mid_ch)
+    a_weights = torch.zeros((P, 1), dtype=torch.float32, device=dev) if training else None
+    p.training = int(bool(training))
+    p.out_rgb, p.out_dpt, p.out_acc = out_rgb.data_ptr(), out_dpt.data_ptr(), out_acc.data_ptr()
+    p.out_norm, p.out_dist, p.out_aux = out_norm.data_ptr(), out_dist.data_ptr(), out_aux.data_ptr()
+    p.mid_val = mid_val.data_ptr()
+    p.a_weights = _ptr(a_weights)
+    p.counters = _ptr(counters)
+    _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))
+    del keep
+    return out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights
+
+
+def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, background, means3D, shs, degree,
+                           colors_precomp, others_precomp, opacities, scales, scale_modifier, rotations,
+                           transMat_precomp, viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth,
+                           specular_threshold, out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val,
+                           dL_dout_rgb, dL_dout_dpt, dL_dout_acc, dL_dout_norm, dL_dout_dist, dL_dout_aux):
+    """Reference TraceSurfelsBackwardCUDA (trace_surfels.cpp:307-464): returns (dL_dray_o, dL_dray_d, dL_dmeans3D,
+    dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers, dL_dopacities, dL_dscales, dL_drotations,
+    dL_dtransMat_precomp)."""
+    p, keep = _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp,
+                             others_precomp, opacities, scales, scale_modifier, rotations, max_trace_depth,
+                             specular_threshold, start_from_first)
+    H, W, P, dev = p.H, p.W, p.P, means3D.device
+    saved = [_cuda_f32(x, n) for x, n in ((out_rgb, "out_rgb"), (out_dpt, "out_dpt"), (out_acc, "out_acc"),
+                                          (out_norm, "out_norm"), (out_dist, "out_dist"), (out_aux, "out_aux"),
+                                          (mid_val, "mid_val"))]
+    mid_ch = (14 + p.aux) * (p.mtd_alloc + 1)
+    if saved[6].numel() != H * W * mid_ch or saved[5].numel() != H * W * p.aux:
+        raise RuntimeError("mid_val / out_aux do not match the settings they were traced with")
+    p.out_rgb, p.out_dpt, p.out_acc, p.out_norm, p.out_dist, p.out_aux, p.mid_val = [x.data_ptr() for x in saved]
+    ups = [_cuda_f32(x, n) for x, n in ((dL_dout_rgb, "dL_dout_rgb"), (dL_dout_dpt, "dL_dout_dpt"),
+                                        (dL_dout_acc, "dL_dout_acc"), (dL_dout_norm, "dL_dout_norm"),
+                                        (dL_dout_dist, "dL_dout_dist"), (dL_dout_aux, "dL_dout_aux"))]
+    want = (3, 1, 1, 3, None, p.aux)
+    for x, ch, n in zip(ups, want, ("rgb", "dpt", "acc", "norm", "dist", "aux")):
+        if ch is not None and x.numel() != H * W * ch:
+            raise RuntimeError("upstream gradient of %s has the wrong size" % n)
+    p.dL_drgb, p.dL_ddpt, p.dL_dacc, p.dL_dnorm, p.dL_ddist, p.dL_daux = (
+        ups[0].data_ptr(), ups[1].data_ptr(), ups[2].data_ptr(), ups[3].data_ptr(), _ptr(ups[4]), ups[5].data_ptr())
+    zeros = lambda *shape: torch.zeros(shape, dtype=torch.float32, device=dev)  # noqa: E731 (atomically accumulated)
+    dL_dray_o = torch.empty((H, W, 3), dtype=torch.float32, device=dev)
+    dL_dray_d = torch.empty((H, W, 3), dtype=torch.float32, device=dev)
+    dL_dmeans3D, dL_dgrads3D, dL_dgrads3D_abs = zeros(P, 3), zeros(P, 3), zeros(P, 3)
+    dL_dshs, dL_dcolors, dL_dothers = zeros(P, p.M, 3), zeros(P, NUM_CHANNELS), zeros(P, p.aux)
+    dL_dopacities, dL_dscales, dL_drotations = zeros(P, 1), zeros(P, 2), zeros(P, 4)
+    dL_dtransMat = zeros(P, 9)
+    p.dL_dray_o, p.dL_dray_d = dL_dray_o.data_ptr(), dL_dray_d.data_ptr()
+    p.dL_dmeans3D, p.dL_dgrads3D, p.dL_dshs = dL_dmeans3D.data_ptr(), dL_dgrads3D.data_ptr(), _ptr(dL_dshs)
+    p.dL_dcolors, p.dL_dothers = dL_dcolors.data_ptr(), dL_dothers.data_ptr()
+    p.dL_dopacities, p.dL_dscales, p.dL_drotations = (dL_dopacities.data_ptr(), dL_dscales.data_ptr(),
+                                                      dL_drotations.data_ptr())
+    _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))
+    del keep
+    return (dL_dray_o, dL_dray_d, dL_dmeans3D, dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers,
+            dL_dopacities, dL_dscales, dL_drotations, dL_dtransMat)

@@ -1,0 +1,148 @@
+/*
+ * C ABI of the MI355X surfel ray tracer (libdst.so).
+ *
+ * Plain pointers and sizes only: every pointer in DstParams is a DEVICE pointer
+ * to fp32 data (int32 for the triangle indices), laid out exactly like the
+ * tensors of the reference launcher.  `stream` is a hipStream_t passed as
+ * void*; all work is enqueued on it and, except where noted, not waited for.
+ * Every entry point returns 0 on success and a nonzero DST_E_* status
+ * otherwise; dst_last_error() then describes the failure.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   ext.cpp:7-12                      pybind module with the four symbols below
+ *   optix_tracer/optix_wrapper.cpp:166-222   OptiXStateWrapper ctor / dtor
+ *   trace_surfels.cpp:36-159          BuildAccelerationStructure
+ *   trace_surfels.cpp:162-304         TraceSurfelsCUDA
+ *   trace_surfels.cpp:307-464         TraceSurfelsBackwardCUDA
+ *   optix_tracer/params.h:21-84       struct Params (launch parameter block)
+ */
+#ifndef DST_API_H
+#define DST_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    DST_OK = 0,
+    DST_E_INVALID = 1,     /* malformed argument (shape, null pointer, out-of-range setting) */
+    DST_E_NO_ACCEL = 2,    /* trace or refit before a successful build */
+    DST_E_TOPOLOGY = 3,    /* triangles are not the two-triangles-per-surfel quads, or refit with another size */
+    DST_E_DEVICE = 4,      /* a HIP runtime call failed */
+    DST_E_UNSUPPORTED = 5  /* setting outside what the kernels are instantiated for */
+};
+
+#define DST_MAX_AUX 8        /* auxiliary channels per surfel (reference AUX_CHANNELS = 2) */
+#define DST_MAX_TRACE_DEPTH 3 /* bounces after the primary ray (reference MAX_TRACE_DEPTH = 1) */
+
+/* Opaque tracer state: owns the acceleration structure and its scratch.
+ * Replaces OptiXStateWrapper (optix_tracer/optix_wrapper.h:25-52). */
+typedef struct dst_ctx dst_ctx;
+
+/* Launch parameter block; mirrors struct Params (optix_tracer/params.h:21-84)
+ * with the compile-time AUX_CHANNELS / MAX_TRACE_DEPTH made runtime fields.
+ * Channel layout of one mid_val slot (optix_tracer/config.h:8-15):
+ * ray_o 0..2, ray_d 3..5, dpt 6, acc 7, norm 8..10, aux 11..11+aux-1, rgb 11+aux..13+aux. */
+typedef struct DstParams {
+    /* sizes and settings */
+    int32_t P, H, W;              /* surfels; ray grid (H,W) = first two dims of ray_o */
+    int32_t D, M;                 /* active SH degree 0..3; coefficients per surfel in shs (0 when colours are given) */
+    int32_t aux;                  /* auxiliary channels, 1..DST_MAX_AUX */
+    int32_t mtd_alloc;            /* mid_val holds mtd_alloc+1 slots per ray */
+    int32_t max_trace_depth;      /* 0..mtd_alloc */
+    int32_t training;             /* accumulate a_weights */
+    int32_t start_from_first;
+    float specular_threshold;
+    float scale_modifier;         /* accepted and ignored, as in the reference device code */
+    /* inputs */
+    const float *ray_o, *ray_d;   /* (H,W,3) */
+    const float *vertices;        /* (4P,3) */
+    const float *background;      /* (3) */
+    const float *means3D;         /* (P,3) */
+    const float *shs;             /* (P,M,3) or NULL */
+    const float *colors_precomp;  /* (P,3) or NULL; exactly one of shs / colors_precomp */
+    const float *others_precomp;  /* (P,aux) or NULL */
+    const float *opacities;       /* (P,1) */
+    const float *scales;          /* (P,2) */
+    const float *rotations;       /* (P,4) quaternion (w,x,y,z) */
+    /* forward outputs, fully written by the kernel (backward reads them) */
+    float *out_rgb;               /* (H,W,3) */
+    float *out_dpt, *out_acc;     /* (H,W,1) */
+    float *out_norm, *out_dist;   /* (H,W,3) */
+    float *out_aux;               /* (H,W,aux) */
+    float *mid_val;               /* (H,W,(mtd_alloc+1)*(14+aux)) */
+    float *a_weights;             /* (P,1), ACCUMULATED into: caller zero-fills; NULL when !training */
+    /* optional forward statistics: counters[0] += entries evaluated, counters[1] += hits composited */
+    unsigned long long *counters;
+    /* upstream gradients (backward) */
+    const float *dL_drgb, *dL_ddpt, *dL_dacc, *dL_ddist, *dL_dnorm, *dL_daux;
+    /* gradient outputs; the per-surfel ones are ACCUMULATED into: caller zero-fills */
+    float *dL_dray_o, *dL_dray_d; /* (H,W,3), fully written */
+    float *dL_dmeans3D, *dL_dgrads3D; /* (P,3) */
+    float *dL_dshs;               /* (P,M,3) */
+    float *dL_dcolors;            /* (P,3) */
+    float *dL_dothers;            /* (P,aux) */
+    float *dL_dopacities;         /* (P,1) */
+    float *dL_dscales;            /* (P,2) */
+    float *dL_drotations;         /* (P,4) */
+} DstParams;
+
+/* Shape of the current acceleration structure, for tests and tools. */
+typedef struct DstAccelInfo {
+    uint32_t n_surfels;    /* leaves */
+    uint32_t n_internal;   /* internal nodes (n_surfels-1, 0 for a single surfel) */
+    uint32_t root;         /* root reference (leaf bit set when n_surfels == 1) */
+    uint32_t node_bytes, leaf_bytes;
+    float scene_lo[3], scene_hi[3]; /* bounds of the quad centroids used for the Morton grid */
+    float max_abs;         /* largest |coordinate| of any vertex */
+    uint32_t builds, refits;
+} DstAccelInfo;
+
+/* Create / destroy the tracer state on the current HIP device.
+ * Replaces OptiXStateWrapper::OptiXStateWrapper / ~OptiXStateWrapper
+ * (optix_tracer/optix_wrapper.cpp:166-222).  dst_create returns NULL on failure. */
+dst_ctx *dst_create(void);
+void dst_destroy(dst_ctx *ctx);
+
+/* Build (rebuild != 0) or refit in place (rebuild == 0) the BVH over the
+ * surfel quads.  vertices: (n_vertices,3) fp32; triangles: (n_triangles,3)
+ * int32 with rows 2g and 2g+1 forming surfel g's quad and sharing an edge
+ * (rows [a,b,c] and [b,c,d]).  A refit reuses the topology of the last build:
+ * n_triangles must be unchanged and `triangles` is not read.  A build waits
+ * for the stream once (it reads back a validity flag); a refit does not.
+ * Replaces BuildAccelerationStructure (trace_surfels.cpp:36-159). */
+int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
+                    uint32_t n_triangles, int rebuild, void *stream);
+
+/* Forward trace: fills out_* and mid_val, accumulates a_weights.
+ * Replaces TraceSurfelsCUDA (trace_surfels.cpp:162-304); stream-ordered, no wait. */
+int dst_trace_forward(dst_ctx *ctx, const DstParams *params, void *stream);
+
+/* Backward re-trace: fills dL_dray_o/d, accumulates the per-surfel gradients.
+ * Replaces TraceSurfelsBackwardCUDA (trace_surfels.cpp:307-464); stream-ordered, no wait. */
+int dst_trace_backward(dst_ctx *ctx, const DstParams *params, void *stream);
+
+/* Message of the last failure on this context (never NULL).  The reference
+ * prints CUDA/OptiX failures and carries on (optix_tracer/common.h:38-50). */
+const char *dst_last_error(dst_ctx *ctx);
+
+/* Introspection for tests: shape of the BVH, and copies of its arrays to HOST
+ * buffers (each may be NULL to skip).  nodes: n_internal*node_bytes, leaves:
+ * n_surfels*leaf_bytes, node_parent: n_internal uint32, leaf_parent: n_surfels
+ * uint32, sorted_keys: n_surfels uint32 Morton codes in leaf order.  Waits for the stream. */
+int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info);
+int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_parent, uint32_t *leaf_parent,
+                       uint32_t *sorted_keys, void *stream);
+
+/* Library version string, and sizeof(DstParams) as compiled (lets a foreign-language binding
+ * verify its own struct layout before the first launch). */
+const char *dst_version(void);
+size_t dst_sizeof_params(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
