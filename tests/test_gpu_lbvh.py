@@ -1,0 +1,143 @@
+"""Structure of the HIP-built LBVH (downloaded through the C ABI) and the error paths of the boundary."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import dst_scenes as S
+
+pytestmark = pytest.mark.gpu
+
+LEAF = 0x80000000
+
+NODE = np.dtype([("lo0", "<f4", 3), ("hi0", "<f4", 3), ("lo1", "<f4", 3), ("hi1", "<f4", 3), ("c0", "<u4"),
+                 ("c1", "<u4"), ("pad", "<u4", 2)])
+LEAFT = np.dtype([("A", "<f4", 3), ("B", "<f4", 3), ("C", "<f4", 3), ("D", "<f4", 3), ("g", "<u4"), ("pad", "<u4", 3)])
+
+
+def download(tracer):
+    import diff_surfel_tracing._C as binding
+    ctx = tracer.optix_context
+    info = ctx.accel_info()
+    assert info.node_bytes == NODE.itemsize == 64 and info.leaf_bytes == LEAFT.itemsize == 64
+    n = info.n_surfels
+    nodes = np.zeros(max(n - 1, 1), NODE)
+    leaves = np.zeros(n, LEAFT)
+    npar, lpar, keys = np.zeros(max(n - 1, 1), np.uint32), np.zeros(n, np.uint32), np.zeros(n, np.uint32)
+    rc = binding.load_library().dst_accel_download(
+        ctx.handle, nodes.ctypes.data, leaves.ctypes.data, npar.ctypes.data, lpar.ctypes.data, keys.ctypes.data,
+        C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    return info, nodes[: n - 1], leaves, npar[: n - 1], lpar, keys
+
+
+def check_tree(info, nodes, leaves, npar, lpar, keys, vertices):
+    n = info.n_surfels
+    assert (np.diff(keys.astype(np.int64)) >= 0).all()                 # Morton order
+    assert sorted(leaves["g"].tolist()) == list(range(n))              # every surfel exactly once
+    V = vertices.reshape(n, 4, 3)
+    for name, k in (("A", 0), ("B", 1), ("C", 2), ("D", 3)):
+        np.testing.assert_array_equal(leaves[name], V[leaves["g"], k])
+    llo = np.minimum.reduce([leaves[c] for c in "ABCD"])
+    lhi = np.maximum.reduce([leaves[c] for c in "ABCD"])
+    # walk from the root: every node and leaf reached once, parents consistent, boxes = exact union of content
+    seen_nodes, seen_leaves = np.zeros(n - 1, bool), np.zeros(n, bool)
+    box_lo, box_hi = {}, {}
+    stack, order, depth, maxdepth = [(0, 0)], [], {}, 0
+    while stack:
+        i, dep = stack.pop()
+        assert not seen_nodes[i]
+        seen_nodes[i] = True
+        order.append(i)
+        maxdepth = max(maxdepth, dep)
+        for which, c in enumerate((int(nodes["c0"][i]), int(nodes["c1"][i]))):
+            if c & LEAF:
+                j = c & ~LEAF
+                assert not seen_leaves[j] and lpar[j] == ((i << 1) | which)
+                seen_leaves[j] = True
+            else:
+                assert npar[c] == ((i << 1) | which)
+                stack.append((c, dep + 1))
+    assert seen_nodes.all() and seen_leaves.all() and npar[0] == 0xFFFFFFFF
+    assert maxdepth < 62                                                 # the traversal stack holds 64 entries
+    for i in reversed(order):
+        los, his = [], []
+        for c in (int(nodes["c0"][i]), int(nodes["c1"][i])):
+            if c & LEAF:
+                los.append(llo[c & ~LEAF]); his.append(lhi[c & ~LEAF])
+            else:
+                los.append(box_lo[c]); his.append(box_hi[c])
+        np.testing.assert_array_equal(nodes["lo0"][i], los[0]); np.testing.assert_array_equal(nodes["hi0"][i], his[0])
+        np.testing.assert_array_equal(nodes["lo1"][i], los[1]); np.testing.assert_array_equal(nodes["hi1"][i], his[1])
+        box_lo[i], box_hi[i] = np.minimum(los[0], los[1]), np.maximum(his[0], his[1])
+    return maxdepth
+
+
+@pytest.mark.parametrize("maker,P", [(S.scene_cube, 5000), (S.scene_room, 20000), (S.scene_cube, 2), (S.scene_cube, 1025)])
+def test_tree_invariants_after_build_and_refit(tracer, maker, P):
+    sc = maker(P=P, seed=1)
+    v, f = sc["vertices"].cuda(), sc["faces"].cuda()
+    tracer.build_acceleration_structure(v, f, True)
+    info, *arrs = download(tracer)
+    assert info.n_surfels == P and info.n_internal == P - 1
+    cen = 0.5 * (sc["vertices"].reshape(P, 4, 3).amin(1) + sc["vertices"].reshape(P, 4, 3).amax(1)).numpy()
+    np.testing.assert_allclose(list(info.scene_lo), cen.min(0), rtol=0, atol=0)
+    np.testing.assert_allclose(list(info.scene_hi), cen.max(0), rtol=0, atol=0)
+    assert info.max_abs == float(sc["vertices"].abs().max())
+    check_tree(info, *arrs, sc["vertices"].numpy())
+    moved = S.perturb_means(sc, 1, frac=0.5, sigma=0.2)
+    tracer.build_acceleration_structure(moved["vertices"].cuda(), f, False)
+    info2, *arrs2 = download(tracer)
+    np.testing.assert_array_equal(arrs2[1]["g"], arrs[1]["g"])           # refit keeps the leaf order and topology
+    np.testing.assert_array_equal(arrs2[0]["c0"], arrs[0]["c0"])
+    check_tree(info2, *arrs2, moved["vertices"].numpy())
+    assert info2.refits >= 1
+
+
+def test_duplicate_positions_give_a_bounded_tree(tracer):
+    """All centroids in one Morton cell: the hierarchy falls back to index bits and stays balanced."""
+    P = 4096
+    sc = S.scene_cube(P=P, seed=2)
+    sc["means3D"] = torch.zeros(P, 3)
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    tracer.build_acceleration_structure(sc["vertices"].cuda(), sc["faces"].cuda(), True)
+    info, *arrs = download(tracer)
+    depth = check_tree(info, *arrs, sc["vertices"].numpy())
+    assert depth <= 44   # 30 key bits + 12 index bits
+
+
+def test_boundary_errors(tracer):
+    import diff_surfel_tracing as dst
+    sc = S.scene_cube(P=100, seed=0)
+    v, f = sc["vertices"].cuda(), sc["faces"].cuda()
+    fresh = dst.SurfelTracer()
+    with pytest.raises(RuntimeError, match="before any build"):
+        fresh.build_acceleration_structure(v, f, False)
+    bad = f.clone()
+    bad[3, 0] = 0                                                        # second triangle no longer shares the edge
+    with pytest.raises(RuntimeError, match="pairs"):
+        fresh.build_acceleration_structure(v, bad, True)
+    bad = f.clone()
+    bad[0, 2] = 4 * 100 + 7                                              # vertex id out of range
+    with pytest.raises(RuntimeError, match="pairs"):
+        fresh.build_acceleration_structure(v, bad, True)
+    with pytest.raises(RuntimeError, match="2 \\* num_surfels"):
+        fresh.build_acceleration_structure(v, f[:-1], True)
+    fresh.build_acceleration_structure(v, f, True)
+    with pytest.raises(RuntimeError, match="different number of surfels"):
+        fresh.build_acceleration_structure(v[:-4], f[:-2], False)
+    # tracing with another surfel count than the structure holds
+    from helpers import gpu_trace
+    o, d = S.rays_cube(8, 8)
+    other = S.scene_cube(P=50, seed=0)
+    with pytest.raises(RuntimeError, match="differs from the acceleration structure"):
+        gpu_trace(fresh, other, o, d, build=False)
+    with pytest.raises(RuntimeError, match="mtd_alloc|max_trace_depth"):
+        gpu_trace(fresh, sc, o, d, build=False, max_trace_depth=4)
+    wide = S.scene_cube(P=100, seed=0, aux=9)
+    with pytest.raises(RuntimeError, match="aux channels"):
+        gpu_trace(fresh, wide, o, d, build=False)
+    # a failed call leaves the context usable
+    out, _ = gpu_trace(fresh, sc, o, d, build=False)
+    assert np.isfinite(out["rgb"]).all()

@@ -1,0 +1,182 @@
+"""Parity of the HIP path (through the public API and the C ABI underneath) with the CPU oracle on the
+same seeded inputs.  Bar: per-ray forward outputs bit-identical (both sides run the same sequence of
+unfused fp32 operations; the north star asks for 1e-4 absolute), atomically accumulated sums and all
+gradients within 1e-3 of the largest reference magnitude (north star: 1e-3 relative)."""
+import numpy as np
+import pytest
+import torch
+
+import dst_scenes as S
+from helpers import (GRAD_REL, assert_close_sum, assert_forward_exact, gpu_trace, oracle_scene, to_numpy, upstream)
+
+pytestmark = pytest.mark.gpu
+
+
+def check_case(oracle, tracer, scene, ray_o, ray_d, acc_grad=True, grads=True, **kw):
+    """Forward + backward on both sides and compare everything."""
+    H, W = ray_o.shape[:2]
+    s = oracle_scene(oracle, scene, ray_o, ray_d, **kw)
+    ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
+    ug = upstream(H, W, s.aux, acc=acc_grad) if grads else None
+    out, g = gpu_trace(tracer, scene, ray_o, ray_d, upstream=ug, **kw)
+    assert_forward_exact(out, ref)
+    assert_close_sum(out["wet"], ref["wet"], 1e-5, "wet")
+    if grads:
+        refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
+        for k, want in refg.items():
+            if g.get(k) is None:
+                assert k in ("shs", "colors_precomp", "others_precomp"), k
+                continue
+            if np.abs(want).max() == 0:
+                assert np.abs(g[k]).max() == 0, k
+                continue
+            assert_close_sum(g[k], want, GRAD_REL, k)
+    return ref, out
+
+
+def test_config1_cube_sh3(oracle, tracer):
+    """BASELINE config 1: 10k surfels in [-1,1]^3, 128x128 pinhole at distance 3, SH degree 3, depth 0."""
+    sc = S.scene_cube(P=10000, seed=0)
+    ref, _ = check_case(oracle, tracer, sc, *S.rays_cube(128, 128))
+    assert ref["n_con"].max() > 16 and ref["n_proc"].mean() > 10  # several chunks per ray are exercised
+
+
+def test_config1_background_one(oracle, tracer):
+    sc = S.scene_cube(P=10000, seed=0)
+    check_case(oracle, tracer, sc, *S.rays_cube(128, 128, view=1), bg=(1.0, 1.0, 1.0))
+
+
+@pytest.mark.parametrize("aux", [2, 4, 8])
+def test_precomputed_colours_and_aux_channels(oracle, tracer, aux):
+    sc = S.scene_cube(P=4000, seed=10 + aux, colors=True, aux=aux)
+    check_case(oracle, tracer, sc, *S.rays_cube(48, 56, view=2), bg=(0.2, 0.4, 0.6), start_from_first=False)
+
+
+@pytest.mark.parametrize("deg", [0, 1, 2])
+def test_lower_sh_degrees(oracle, tracer, deg):
+    sc = S.scene_cube(P=3000, seed=20 + deg)
+    check_case(oracle, tracer, sc, *S.rays_cube(40, 40), sh_degree=deg)
+
+
+def test_evaluation_mode_returns_zero_weights(oracle, tracer):
+    sc = S.scene_cube(P=1000, seed=3)
+    o, d = S.rays_cube(16, 16)
+    out, _ = gpu_trace(tracer, sc, o, d, training=False)
+    assert out["wet"].shape == (1000,) and (out["wet"] == 0).all()
+    ref = oracle.forward(oracle_scene(oracle, sc, o, d), oracle.HITS_BVH_LEXI)
+    assert_forward_exact(out, ref)
+
+
+@pytest.mark.parametrize("depth,thr", [(1, 0.1), (2, 0.1), (2, 0.45), (3, 0.0)])
+def test_multi_bounce(oracle, tracer, depth, thr):
+    """Config-4 style: reflection rays above specular_threshold, forward and backward through all bounces."""
+    sc = S.scene_room(P=30000, seed=depth, aux=8, half=1.5)
+    sc["others_precomp"][:, 0] = sc["others_precomp"][:, 0] * 0.8 + 0.1   # specular away from 0 (reference divides by it)
+    o, d = S.pinhole_rays(40, 64, 70.0, (-0.6, -0.3, 0.15), (0.9, 0.45, -0.15))
+    ref, _ = check_case(oracle, tracer, sc, o, d, max_trace_depth=depth, specular_threshold=thr)
+    slots = ref["mid"].reshape(40, 64, -1, 22)
+    assert slots.shape[2] == max(depth, 1) + 1
+    reached = (np.abs(slots[:, :, depth, 3:6]).sum(-1) > 0).mean()
+    assert 0.05 < reached  # the deepest bounce is really traced for a good share of the rays
+
+
+def test_thin_ray_lists(oracle, tracer):
+    """(B,P,3) layout with B=1 (config 5's LiDAR rays) and with B=3."""
+    sc = S.scene_lidar(P=20000, seed=1, aux=4)
+    o, d = S.rays_lidar(beams=8, azimuths=256)
+    check_case(oracle, tracer, sc, o, d)
+    o3, d3 = o.reshape(8, 256, 3)[:3].contiguous(), d.reshape(8, 256, 3)[:3].contiguous()
+    check_case(oracle, tracer, sc, o3, d3, grads=False)
+
+
+def test_ragged_image_sizes(oracle, tracer):
+    sc = S.scene_cube(P=2000, seed=5)
+    for H, W in ((37, 53), (1, 1), (9, 7), (64, 1)):
+        check_case(oracle, tracer, sc, *S.rays_cube(H, W))
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 5])
+def test_tiny_scenes(oracle, tracer, P):
+    sc = S.scene_cube(P=P, seed=P)
+    sc["scales"] = sc["scales"] * 8
+    sc["means3D"] = sc["means3D"] * 0.3
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    ref, _ = check_case(oracle, tracer, sc, *S.rays_cube(16, 16))
+    assert ref["n_con"].sum() > 0
+
+
+def test_all_rays_miss(oracle, tracer):
+    sc = S.scene_cube(P=500, seed=2)
+    o, d = S.rays_cube(16, 16)
+    ref, out = check_case(oracle, tracer, sc, o + 10.0, -d, bg=(0.3, 0.2, 0.1))
+    assert (out["acc"] == 0).all() and np.allclose(out["rgb"], [0.3, 0.2, 0.1])
+
+
+def test_coplanar_ties_and_dense_stacks(oracle, tracer):
+    """Exactly equal depths (axis-aligned coplanar quads on a binary grid) and >16 hits per ray: the order must be
+    the oracle's (ascending surfel index), whatever order the BVH delivers them in."""
+    from test_oracle_scalar import _tie_scene
+    sc = _tie_scene(600, seed=3)
+    o = torch.stack(torch.meshgrid(torch.linspace(-0.4, 0.4, 24), torch.linspace(-0.4, 0.4, 24), indexing="ij"), -1)
+    o = torch.cat([o, torch.full((24, 24, 1), 3.0)], -1).contiguous()
+    d = torch.tensor([0.0, 0.0, -1.0]).expand(24, 24, 3).contiguous()
+    ref, _ = check_case(oracle, tracer, sc, o, d)
+    assert ref["n_proc"].max() >= 16
+
+
+def test_refit_equals_rebuild(oracle, tracer):
+    sc = S.scene_lidar(P=30000, seed=2, aux=4)
+    o, d = S.rays_lidar(beams=16, azimuths=128)
+    gpu_trace(tracer, sc, o, d)                       # build on the first frame
+    for frame in (1, 2):
+        moved = S.perturb_means(sc, frame)
+        out_refit, _ = gpu_trace(tracer, moved, o, d, rebuild=False)
+        out_build, _ = gpu_trace(tracer, moved, o, d, rebuild=True)
+        ref = oracle.forward(oracle_scene(oracle, moved, o, d), oracle.HITS_BVH_LEXI)
+        assert_forward_exact(out_refit, ref)
+        assert_forward_exact(out_build, ref)
+
+
+def test_config2_sphere_build_once_then_refit(oracle, tracer):
+    sc = S.scene_sphere(P=100000, seed=0)
+    for view in range(3):
+        o, d = S.rays_sphere(96, 96, view=view)
+        s = oracle_scene(oracle, sc, o, d)
+        ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
+        out, _ = gpu_trace(tracer, sc, o, d, rebuild=(view == 0))
+        assert_forward_exact(out, ref)
+        assert ref["acc"].mean() > 0.2
+
+
+def test_debug_flag_and_saved_tensor_reuse(oracle, tracer):
+    sc = S.scene_cube(P=800, seed=9)
+    o, d = S.rays_cube(16, 16)
+    out, _ = gpu_trace(tracer, sc, o, d, debug=True, upstream=upstream(16, 16, 2))
+    ref = oracle.forward(oracle_scene(oracle, sc, o, d), oracle.HITS_BVH_LEXI)
+    assert_forward_exact(out, ref)
+
+
+def test_config3_full_size_properties_and_sampled_parity(oracle, tracer):
+    """BASELINE config 3 at its real size (1M surfels, 1920x1080): size-independent invariants on the whole
+    image, run-to-run determinism, and bit parity with the oracle on a sample of 4096 pixels."""
+    dev = "cuda"
+    sc = S.scene_room(P=1000000, seed=0)
+    o, d = S.rays_room(1080, 1920)
+    out, _ = gpu_trace(tracer, sc, o, d)
+    acc = out["acc"].astype(np.float64)
+    assert np.isfinite(out["rgb"]).all() and (acc >= 0).all() and (acc <= 1).all()
+    np.testing.assert_allclose(acc.sum(), out["wet"].astype(np.float64).sum(), rtol=1e-4)   # checksum of checksums
+    np.testing.assert_array_equal(out["mid"][..., 13:16], out["rgb"])                       # bg = 0, depth 0
+    np.testing.assert_array_equal(out["mid"][..., 16:], 0)
+    out2, _ = gpu_trace(tracer, sc, o, d, build=False)
+    for k in ("rgb", "dpt", "acc", "norm", "mid"):
+        np.testing.assert_array_equal(out[k], out2[k])
+    gen = torch.Generator().manual_seed(5)
+    pick = torch.randperm(1080 * 1920, generator=gen)[:4096]
+    so, sd = o.reshape(-1, 3)[pick].reshape(64, 64, 3).contiguous(), d.reshape(-1, 3)[pick].reshape(64, 64, 3).contiguous()
+    ref = oracle.forward(oracle_scene(oracle, sc, so, sd), oracle.HITS_BVH_LEXI)
+    for k in ("rgb", "dpt", "acc", "norm"):
+        got = out[k].reshape(1080 * 1920, -1)[pick.numpy()].reshape(ref[k].shape)
+        np.testing.assert_array_equal(got.view(np.uint32), ref[k].view(np.uint32), err_msg=k)
+    assert ref["n_con"].mean() > 10
+    del dev
