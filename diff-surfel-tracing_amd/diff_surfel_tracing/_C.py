@@ -179,9 +179,11 @@ def _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, col
 def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, background, means3D, shs, degree,
                   colors_precomp, others_precomp, opacities, scales, scale_modifier, rotations, transMat_precomp,
                   viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth, specular_threshold,
-                  counters=None):
+                  counters=None, events=None):
     """Reference TraceSurfelsCUDA (trace_surfels.cpp:162-304): returns
-    (out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights or None)."""
+    (out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights or None).
+    Extras for measurement: `counters` (2 int64 on the device) receives the evaluated / composited hit totals;
+    `events` (two torch.cuda.Event) are recorded on the launch stream right around the kernel launch."""
     p, keep = _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp,
                              others_precomp, opacities, scales, scale_modifier, rotations, max_trace_depth,
                              specular_threshold, start_from_first)
@@ -197,7 +199,11 @@ def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, backg
     p.mid_val = mid_val.data_ptr()
     p.a_weights = _ptr(a_weights)
     p.counters = _ptr(counters)
+    if events is not None:
+        events[0].record()
     _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))
+    if events is not None:
+        events[1].record()
     del keep
     return out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights
 
@@ -206,7 +212,8 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
                            colors_precomp, others_precomp, opacities, scales, scale_modifier, rotations,
                            transMat_precomp, viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth,
                            specular_threshold, out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val,
-                           dL_dout_rgb, dL_dout_dpt, dL_dout_acc, dL_dout_norm, dL_dout_dist, dL_dout_aux):
+                           dL_dout_rgb, dL_dout_dpt, dL_dout_acc, dL_dout_norm, dL_dout_dist, dL_dout_aux,
+                           events=None):
     """Reference TraceSurfelsBackwardCUDA (trace_surfels.cpp:307-464): returns (dL_dray_o, dL_dray_d, dL_dmeans3D,
     dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers, dL_dopacities, dL_dscales, dL_drotations,
     dL_dtransMat_precomp)."""
@@ -242,7 +249,11 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
     p.dL_dcolors, p.dL_dothers = dL_dcolors.data_ptr(), dL_dothers.data_ptr()
     p.dL_dopacities, p.dL_dscales, p.dL_drotations = (dL_dopacities.data_ptr(), dL_dscales.data_ptr(),
                                                       dL_drotations.data_ptr())
+    if events is not None:
+        events[0].record()
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))
+    if events is not None:
+        events[1].record()
     del keep
     return (dL_dray_o, dL_dray_d, dL_dmeans3D, dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers,
             dL_dopacities, dL_dscales, dL_drotations, dL_dtransMat)

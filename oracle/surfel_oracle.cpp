@@ -59,6 +59,7 @@
 #include <cstring>
 #include <vector>
 #include <algorithm>
+#include <chrono>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
@@ -918,6 +919,7 @@ int oracle_trace_forward(const OracleParams *p) {
     Accum acc;
     if (p->training && p->a_weights) acc.w.assign((size_t)p->P, 0.0);
     Accum *accp = (p->training && p->a_weights) ? &acc : nullptr;
+    const auto t_start = std::chrono::steady_clock::now();
 #pragma omp parallel for schedule(dynamic, 64)
     for (long r = 0; r < R; ++r) {
         V3 o = ld3(p->ray_o + 3 * r), d = ld3(p->ray_d + 3 * r);
@@ -938,6 +940,8 @@ int oracle_trace_forward(const OracleParams *p) {
         if (p->n_proc) p->n_proc[r] = n_proc;
         if (p->n_con) p->n_con[r] = n_con;
     }
+    if (p->trace_seconds)
+        *p->trace_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_start).count();
     if (accp) flush(acc.w, p->a_weights);
     return 0;
 }
@@ -958,6 +962,7 @@ int oracle_trace_backward(const OracleParams *p) {
     acc.opac.assign(P, 0.0);
     acc.scales.assign(P * 2, 0.0);
     acc.rots.assign(P * 4, 0.0);
+    const auto t_start = std::chrono::steady_clock::now();
 #pragma omp parallel for schedule(dynamic, 64)
     for (long r = 0; r < R; ++r) {
         float g_aux[kMaxAux] = {0};
@@ -968,6 +973,8 @@ int oracle_trace_backward(const OracleParams *p) {
         p->dL_dray_o[3 * r + 0] = g_o.x; p->dL_dray_o[3 * r + 1] = g_o.y; p->dL_dray_o[3 * r + 2] = g_o.z;
         p->dL_dray_d[3 * r + 0] = g_d.x; p->dL_dray_d[3 * r + 1] = g_d.y; p->dL_dray_d[3 * r + 2] = g_d.z;
     }
+    if (p->trace_seconds)
+        *p->trace_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_start).count();
     flush(acc.means, p->dL_dmeans3D);
     flush(acc.grads, p->dL_dgrads3D);
     flush(acc.shs, p->dL_dshs);

@@ -56,6 +56,7 @@ typedef struct OracleParams {
     float *a_weights;             /* (P) or NULL */
     /* optional per-ray counters (forward): entries that reach the uv evaluation / composited hits */
     int32_t *n_proc, *n_con;      /* (H*W) or NULL */
+    double *trace_seconds;        /* optional: wall time of the ray loop alone (set-up and CPU BVH build excluded) */
     /* upstream gradients */
     const float *dL_drgb, *dL_ddpt, *dL_dacc, *dL_ddist, *dL_dnorm, *dL_daux;
     /* gradient outputs */

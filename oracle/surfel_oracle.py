@@ -30,7 +30,7 @@ class OracleParams(C.Structure):
                               "scales", "rotations")]
         + [(n, _FP) for n in ("out_rgb", "out_dpt", "out_acc", "out_norm", "out_dist", "out_aux", "mid_val",
                               "a_weights")]
-        + [("n_proc", _IP), ("n_con", _IP)]
+        + [("n_proc", _IP), ("n_con", _IP), ("trace_seconds", C.POINTER(C.c_double))]
         + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
         + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
                               "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
@@ -137,9 +137,12 @@ def forward(sc, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0, coun
     p.a_weights = _fp(out["wet"]) if sc.training else None
     if counters:
         p.n_proc, p.n_con = _ip(out["n_proc"]), _ip(out["n_con"])
+    secs = C.c_double(0.0)
+    p.trace_seconds = C.pointer(secs)
     rc = lib().oracle_trace_forward(C.byref(p))
     if rc:
         raise RuntimeError("oracle_trace_forward failed with status %d" % rc)
+    sc.trace_seconds = secs.value  # wall time of the ray loop of this call
     return out
 
 
@@ -167,9 +170,12 @@ def backward(sc, fwd, grads, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_th
     p.dL_dmeans3D, p.dL_dgrads3D, p.dL_dshs = _fp(out["means3D"]), _fp(out["grads3D"]), _fp(out["shs"])
     p.dL_dcolors, p.dL_dothers = _fp(out["colors_precomp"]), _fp(out["others_precomp"])
     p.dL_dopacities, p.dL_dscales, p.dL_drotations = _fp(out["opacities"]), _fp(out["scales"]), _fp(out["rotations"])
+    secs = C.c_double(0.0)
+    p.trace_seconds = C.pointer(secs)
     rc = lib().oracle_trace_backward(C.byref(p))
     if rc:
         raise RuntimeError("oracle_trace_backward failed with status %d" % rc)
+    sc.trace_seconds = secs.value  # wall time of the ray loop of this call
     return out
 
 
