@@ -74,7 +74,7 @@ int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, co
     const uint32_t P = n_triangles / 2;
     if ((uint64_t)n_vertices < 4ull * P)
         return dst_fail(ctx, DST_E_TOPOLOGY, "vertices must hold four corners per surfel (4 * num_surfels, 3)");
-    if (P > 0x7FFFFFFFu / 4u) return dst_fail(ctx, DST_E_UNSUPPORTED, "too many surfels");
+    if (P > DST_MAX_SURFELS) return dst_fail(ctx, DST_E_UNSUPPORTED, "too many surfels");
     if (rebuild) {
         if (!triangles) return dst_fail(ctx, DST_E_INVALID, "triangles must have dimensions (num_triangles, 3)");
     } else {
@@ -113,7 +113,7 @@ int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info) {
     if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "no acceleration structure");
     info->n_surfels = ctx->n_leaves;
     info->n_internal = ctx->n_leaves - 1;
-    info->root = (ctx->n_leaves == 1) ? DST_LEAF_BIT : 0u;
+    info->root = dst_root_ref(ctx->n_leaves);
     info->node_bytes = sizeof(DstNode);
     info->leaf_bytes = sizeof(DstLeaf);
     for (int a = 0; a < 3; ++a) {

@@ -11,13 +11,29 @@
 #define DST_NO_PARENT 0xFFFFFFFFu
 #define DST_WAVE 64
 
-// Internal node of the binary BVH: the boxes of both children live in the parent, so one
-// 64-byte wave-uniform fetch decides both descents.
+#define DST_GROUP 4            // quads per leaf group (a subtree of at most this many leaves is tested as a unit)
+#define DST_WIDE 4             // children per traversal node
+#define DST_REF_FIRST_MASK 0x0FFFFFFFu   // leaf-group reference: DST_LEAF_BIT | (count-1) << 28 | first leaf position
+#define DST_MAX_SURFELS 0x0FFFFFFFu
+
+// Internal node of the binary hierarchy (Karras): the boxes of both children live in the parent.
+// The builder and the refit work on these; the trace kernels read the 4-wide nodes derived from them.
 struct alignas(64) DstNode {
     float lo0[3], hi0[3];
     float lo1[3], hi1[3];
-    uint32_t c0, c1;  // child references: DST_LEAF_BIT | leaf position, or internal node index
-    uint32_t pad[2];
+    uint32_t c0, c1;      // child references: DST_LEAF_BIT | leaf position, or internal node index
+    uint32_t first, last; // range of leaf positions below this node
+};
+
+// Traversal node, indexed like the binary node it was collapsed from: up to four children (the binary
+// node's grandchildren, or a child itself where that child is a leaf group), boxes stored by coordinate.
+// One 128-byte wave-uniform fetch decides four descents.
+struct alignas(128) DstWideNode {
+    float lox[DST_WIDE], loy[DST_WIDE], loz[DST_WIDE];
+    float hix[DST_WIDE], hiy[DST_WIDE], hiz[DST_WIDE];
+    uint32_t ref[DST_WIDE];   // wide node index, or leaf-group reference
+    uint32_t count;           // children in use (2..4)
+    uint32_t pad[3];
 };
 
 // Leaf = one surfel quad in Morton order: corners A,B,C,D (triangles ABC and BCD) and the surfel id.
@@ -35,7 +51,7 @@ struct DstBounds {          // device-resident reduction targets, order-preservi
 
 // Device-side view of the acceleration structure handed to the trace kernels.
 struct DstAccelView {
-    const DstNode *nodes;
+    const DstWideNode *wide;
     const DstLeaf *leaves;
     const DstBounds *bounds;  // max_abs sizes the conservative slab padding; read on the device so that a
                               // refit never needs a host round trip
@@ -52,6 +68,7 @@ struct dst_ctx {
     bool built = false;
     uint32_t builds = 0, refits = 0;
     DstNode *nodes = nullptr;
+    DstWideNode *wide = nullptr;
     DstLeaf *leaves = nullptr;
     uint32_t *node_parent = nullptr, *leaf_parent = nullptr;  // (parent << 1) | which child
     uint32_t *flags = nullptr;                                // arrival counters of the bottom-up fit
@@ -64,6 +81,11 @@ struct dst_ctx {
     DstBounds *bounds_host = nullptr;  // pinned host copy
     float scene_lo[3] = {0, 0, 0}, scene_hi[3] = {0, 0, 0}, max_abs = 0;
 };
+
+// Where a traversal starts: the wide node of the binary root, or one leaf group when the scene is that small.
+static inline uint32_t dst_root_ref(uint32_t n_leaves) {
+    return n_leaves <= DST_GROUP ? (DST_LEAF_BIT | ((n_leaves - 1u) << 28)) : 0u;
+}
 
 // lbvh.hip
 int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,

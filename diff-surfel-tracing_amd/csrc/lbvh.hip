@@ -270,8 +270,8 @@ __global__ void k_karras(const uint32_t *__restrict__ keys, DstNode *__restrict_
     }
     nodes[i].c0 = c0;
     nodes[i].c1 = c1;
-    nodes[i].pad[0] = 0;
-    nodes[i].pad[1] = 0;
+    nodes[i].first = (uint32_t)lo;
+    nodes[i].last = (uint32_t)hi;
     if (i == 0) node_parent[0] = DST_NO_PARENT;
 }
 
@@ -333,6 +333,53 @@ __global__ void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
     }
 }
 
+// Reference the trace kernels follow for a child of a binary node: a subtree of at most DST_GROUP leaves
+// (contiguous in Morton order) is one leaf group, anything larger is the wide node of the same index.
+__device__ __forceinline__ uint32_t traversal_ref(const DstNode *__restrict__ nodes, uint32_t c) {
+    if (c & DST_LEAF_BIT) return DST_LEAF_BIT | (c & DST_REF_FIRST_MASK);
+    const uint32_t first = nodes[c].first, count = nodes[c].last - first + 1u;
+    if (count <= DST_GROUP) return DST_LEAF_BIT | ((count - 1u) << 28) | first;
+    return c;
+}
+
+// Collapse the fitted binary hierarchy into 4-wide traversal nodes: node i offers its grandchildren, except
+// that a child which is already a leaf group is offered itself.
+__global__ void k_widen(const DstNode *__restrict__ nodes, DstWideNode *__restrict__ wide, uint32_t n_internal) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_internal) return;
+    const DstNode nd = nodes[i];
+    if (nd.last - nd.first + 1u <= DST_GROUP) return;   // inside a leaf group: never visited
+    DstWideNode w;
+    uint32_t k = 0;
+    auto put = [&](const float *lo, const float *hi, uint32_t ref) {
+        w.lox[k] = lo[0]; w.loy[k] = lo[1]; w.loz[k] = lo[2];
+        w.hix[k] = hi[0]; w.hiy[k] = hi[1]; w.hiz[k] = hi[2];
+        w.ref[k] = ref;
+        ++k;
+    };
+    const uint32_t cs[2] = {nd.c0, nd.c1};
+    const float *los[2] = {nd.lo0, nd.lo1}, *his[2] = {nd.hi0, nd.hi1};
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        const uint32_t r = traversal_ref(nodes, cs[s]);
+        if (r & DST_LEAF_BIT) {
+            put(los[s], his[s], r);
+        } else {
+            const DstNode ch = nodes[cs[s]];
+            put(ch.lo0, ch.hi0, traversal_ref(nodes, ch.c0));
+            put(ch.lo1, ch.hi1, traversal_ref(nodes, ch.c1));
+        }
+    }
+    w.count = k;
+    for (; k < DST_WIDE; ++k) {   // unused slots: the traversal masks them by `count`
+        w.lox[k] = w.loy[k] = w.loz[k] = 0.f;
+        w.hix[k] = w.hiy[k] = w.hiz[k] = 0.f;
+        w.ref[k] = DST_LEAF_BIT;  // would be a harmless one-quad group, never another node
+    }
+    w.pad[0] = w.pad[1] = w.pad[2] = 0u;
+    wide[i] = w;
+}
+
 inline dim3 grid_for(uint32_t n, int block = kBlock) { return dim3((n + block - 1) / block); }
 
 int ensure_capacity(dst_ctx *ctx, uint32_t P) {
@@ -341,6 +388,7 @@ int ensure_capacity(dst_ctx *ctx, uint32_t P) {
     const size_t n = P;
     const size_t tiles = (n + kTile - 1) / kTile;
     DST_HIP(ctx, hipMalloc((void **)&ctx->nodes, sizeof(DstNode) * std::max<size_t>(n - 1, 1)));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->wide, sizeof(DstWideNode) * std::max<size_t>(n - 1, 1)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->leaves, sizeof(DstLeaf) * n));
     DST_HIP(ctx, hipMalloc((void **)&ctx->node_parent, sizeof(uint32_t) * n));
     DST_HIP(ctx, hipMalloc((void **)&ctx->leaf_parent, sizeof(uint32_t) * n));
@@ -367,6 +415,7 @@ void dst_lbvh_free(dst_ctx *ctx) {
         p = nullptr;
     };
     rel(ctx->nodes);
+    rel(ctx->wide);
     rel(ctx->leaves);
     rel(ctx->node_parent);
     rel(ctx->leaf_parent);
@@ -431,6 +480,8 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->flags, 0u, n);
     hipLaunchKernelGGL(k_fit, grid_for(n), dim3(kBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
                        ctx->flags, ctx->leaves, n);
+    if (n > DST_GROUP)
+        hipLaunchKernelGGL(k_widen, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, ctx->wide, n - 1);
     DST_HIP(ctx, hipGetLastError());
 
     if (rebuild) {

@@ -184,91 +184,143 @@ __device__ __forceinline__ bool slab_hit(const RaySlab &s, const uint32_t *box /
     return tn <= tf;
 }
 
-// The (t, idx) pairs of the 16 nearest hits, ascending; ties in t resolved by ascending idx so that
-// the content does not depend on the order in which the BVH delivers candidates.
+// The 16 nearest hits of a lane, ascending.  One entry = (bits of t) << 32 | idx: t is positive, so the
+// unsigned 64-bit order is the (t, idx) lexicographic order and the content does not depend on the order in
+// which the BVH delivers candidates (ties in t resolve to ascending primitive index).
 struct KBuf {
-    float t[kChunk];
-    uint32_t i[kChunk];
+    uint64_t e[kChunk];
 };
+__device__ __forceinline__ uint64_t kb_pack(float t, uint32_t idx) { return ((uint64_t)__float_as_uint(t) << 32) | idx; }
+__device__ __forceinline__ float kb_t(uint64_t e) { return __uint_as_float((uint32_t)(e >> 32)); }
+__device__ __forceinline__ uint32_t kb_idx(uint64_t e) { return (uint32_t)e; }
 
 __device__ __forceinline__ void kbuf_reset(KBuf &b) {
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) {
-        b.t[k] = kInfDepth;
-        b.i[k] = 0u;
-    }
+    for (int k = 0; k < kChunk; ++k) b.e[k] = kb_pack(kInfDepth, 0u);
 }
 
-__device__ __forceinline__ void kbuf_insert(KBuf &b, float t, uint32_t idx, bool on) {
-    float ct = t;
-    uint32_t ci = idx;
+// Sorted insert in place: slot k keeps its entry if that is smaller than the new one, else takes the new one
+// (if the slot above kept its entry) or the entry from the slot above.
+__device__ __forceinline__ void kbuf_insert(KBuf &b, uint64_t x, bool on) {
+    bool keep_k = b.e[kChunk - 1] < x;
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) {
-        bool sw = on && ((ct < b.t[k]) || (ct == b.t[k] && ci < b.i[k]));
-        float tt = b.t[k];
-        uint32_t ti = b.i[k];
-        b.t[k] = sw ? ct : tt;
-        b.i[k] = sw ? ci : ti;
-        ct = sw ? tt : ct;
-        ci = sw ? ti : ci;
+    for (int k = kChunk - 1; k >= 1; --k) {
+        const bool keep_up = b.e[k - 1] < x;
+        const uint64_t in = keep_up ? x : b.e[k - 1];
+        b.e[k] = (on && !keep_k) ? in : b.e[k];
+        keep_k = keep_up;
+    }
+    b.e[0] = (on && !keep_k) ? x : b.e[0];
+}
+
+#ifdef DST_STATS
+struct WaveStats { unsigned long long nodes, leaves, t_trav, t_comp, chunks, leaf_any; };
+#define STAT(x) x
+#else
+#define STAT(x)
+#endif
+
+// Test all lanes' rays against one quad record and admit the hits into the lanes' buffers.
+__device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
+#ifdef DST_STATS
+                                          , WaveStats &ws
+#endif
+) {
+    uint32_t L[13];
+    load_uniform<13>(leaf, L);
+    STAT(ws.leaves++;)
+    F3 A = f3(__uint_as_float(L[0]), __uint_as_float(L[1]), __uint_as_float(L[2]));
+    F3 B = f3(__uint_as_float(L[3]), __uint_as_float(L[4]), __uint_as_float(L[5]));
+    F3 C = f3(__uint_as_float(L[6]), __uint_as_float(L[7]), __uint_as_float(L[8]));
+    F3 Dv = f3(__uint_as_float(L[9]), __uint_as_float(L[10]), __uint_as_float(L[11]));
+    float t = 0.f;
+    uint32_t tri = 0u;
+    const bool hit = active && ray_quad(o, d, A, B, C, Dv, t, tri);
+    const uint64_t x = kb_pack(t, 2u * L[12] + tri);
+    const bool adm = hit && (x < buf.e[kChunk - 1]);
+    if (__ballot(adm) != 0ull) {
+        STAT(ws.leaf_any++;)
+        cnt += adm ? 1u : 0u;
+        kbuf_insert(buf, x, adm);
     }
 }
 
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
-// to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow.
+// to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow: nodes and quads
+// are fetched once per wave, the stack is three VGPRs addressed by lane (192 entries: the binary hierarchy
+// is at most 62 levels deep and each 4-wide step defers at most three children).
 __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
-                                           uint32_t &cnt) {
-    if (__ballot(active) == 0ull) return;
+                                           uint32_t &cnt
+#ifdef DST_STATS
+                                           , WaveStats &ws
+#define WSP , ws
+#else
+#define WSP
+#endif
+) {
+    const uint64_t live = __ballot(active);
+    if (live == 0ull) return;
     const RaySlab slab = make_slab(o, d, max_abs);
     const uint32_t lane = __lane_id();
-    uint32_t stack = 0u;  // entry k lives in lane k; the tree is at most 62 levels deep (30-bit keys + index bits)
+    const int rep = __builtin_ctzll(live);   // the lane whose entry distances order the children
+    uint32_t stack0 = 0u, stack1 = 0u, stack2 = 0u;
     int sp = 0;
     uint32_t ref = acc.root;
-    for (;;) {
+    // A well-formed hierarchy is walked in at most one step per node and per leaf group; the cap makes the
+    // loop finite whatever the memory holds.
+    for (uint32_t budget = 2u * acc.n_leaves + 8u; budget != 0u; --budget) {
         if (ref & DST_LEAF_BIT) {
-            uint32_t L[13];
-            load_uniform<13>(&acc.leaves[ref & ~DST_LEAF_BIT], L);
-            F3 A = f3(__uint_as_float(L[0]), __uint_as_float(L[1]), __uint_as_float(L[2]));
-            F3 B = f3(__uint_as_float(L[3]), __uint_as_float(L[4]), __uint_as_float(L[5]));
-            F3 C = f3(__uint_as_float(L[6]), __uint_as_float(L[7]), __uint_as_float(L[8]));
-            F3 Dv = f3(__uint_as_float(L[9]), __uint_as_float(L[10]), __uint_as_float(L[11]));
-            float t = 0.f;
-            uint32_t tri = 0u;
-            bool hit = active && ray_quad(o, d, A, B, C, Dv, t, tri);
-            uint32_t idx = 2u * L[12] + tri;
-            bool adm = hit && ((t < buf.t[kChunk - 1]) || (t == buf.t[kChunk - 1] && idx < buf.i[kChunk - 1]));
-            if (__ballot(adm) != 0ull) {
-                cnt += adm ? 1u : 0u;
-                kbuf_insert(buf, t, idx, adm);
-            }
-            if (sp == 0) break;
-            --sp;
-            ref = __builtin_amdgcn_readlane(stack, sp);
+            const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
+            for (uint32_t q = 0; q < count && first + q < acc.n_leaves; ++q)
+                test_leaf(&acc.leaves[first + q], o, d, active, buf, cnt WSP);
         } else {
-            uint32_t Nd[14];
-            load_uniform<14>(&acc.nodes[ref], Nd);
-            const float tmax = active ? buf.t[kChunk - 1] : -1.0f;
-            float tn0, tn1;
-            bool h0 = slab_hit(slab, &Nd[0], tmax, tn0);
-            bool h1 = slab_hit(slab, &Nd[6], tmax, tn1);
-            const uint64_t b0 = __ballot(h0), b1 = __ballot(h1);
-            if ((b0 | b1) == 0ull) {
-                if (sp == 0) break;
-                --sp;
-                ref = __builtin_amdgcn_readlane(stack, sp);
-            } else if (b0 != 0ull && b1 != 0ull) {
-                // both wanted: the side most lanes enter first goes first, the other is deferred
-                int v1 = __popcll(__ballot(h1 && (!h0 || tn1 < tn0)));
-                int v0 = __popcll(__ballot(h0 && (!h1 || tn0 <= tn1)));
-                uint32_t near = (v1 > v0) ? Nd[13] : Nd[12];
-                uint32_t far = (v1 > v0) ? Nd[12] : Nd[13];
-                stack = (lane == (uint32_t)sp) ? far : stack;  // entry sp lives in lane sp
-                ++sp;
-                ref = near;
-            } else {
-                ref = (b0 != 0ull) ? Nd[12] : Nd[13];
+            if (ref + 1u >= acc.n_leaves) break;   // not a node of this hierarchy
+            uint32_t Nd[29];
+            load_uniform<29>(&acc.wide[ref], Nd);
+            STAT(ws.nodes++;)
+            const float tmax = active ? kb_t(buf.e[kChunk - 1]) : -1.0f;
+            const uint32_t n_child = Nd[28];
+            uint32_t key[DST_WIDE], cref[DST_WIDE];
+            int n_push = 0;
+#pragma unroll
+            for (int k = 0; k < DST_WIDE; ++k) {
+                const uint32_t box[6] = {Nd[k], Nd[4 + k], Nd[8 + k], Nd[12 + k], Nd[16 + k], Nd[20 + k]};
+                float tn;
+                const bool h = slab_hit(slab, box, tmax, tn) && (uint32_t)k < n_child;   // unused slots are never entered
+                const bool any = __ballot(h) != 0ull;
+                // entry distance of the representative lane (non-negative, so its bits order like the value)
+                const uint32_t kk = __builtin_amdgcn_readlane(h ? __float_as_uint(tn) : 0x7F800000u, rep);
+                key[k] = any ? kk : 0xFFFFFFFFu;
+                cref[k] = Nd[24 + k];
+                n_push += any ? 1 : 0;
+            }
+            if (n_push > 0) {
+                // sort the four (key, ref) pairs, nearest first; children nobody wants carry the largest key
+#define CSWAP(a, b)                                                            \
+    {                                                                          \
+        const bool sw_ = key[b] < key[a];                                      \
+        const uint32_t ka_ = sw_ ? key[b] : key[a], kb_ = sw_ ? key[a] : key[b]; \
+        const uint32_t ra_ = sw_ ? cref[b] : cref[a], rb_ = sw_ ? cref[a] : cref[b]; \
+        key[a] = ka_; key[b] = kb_; cref[a] = ra_; cref[b] = rb_;              \
+    }
+                CSWAP(0, 1) CSWAP(2, 3) CSWAP(0, 2) CSWAP(1, 3) CSWAP(1, 2)
+#undef CSWAP
+                // defer the farther ones (farthest first), continue with the nearest
+                for (int k = n_push - 1; k >= 1; --k) {
+                    const uint32_t v = cref[k];
+                    const uint32_t slot = (uint32_t)sp & 63u;
+                    if (sp < 64) stack0 = (lane == slot) ? v : stack0;
+                    else if (sp < 128) stack1 = (lane == slot) ? v : stack1;
+                    else stack2 = (lane == slot) ? v : stack2;
+                    ++sp;
+                }
+                ref = cref[0];
+                continue;
             }
         }
+        if (sp == 0) break;
+        --sp;
+        ref = __builtin_amdgcn_readlane(sp < 64 ? stack0 : (sp < 128 ? stack1 : stack2), sp & 63);
     }
 }
 
@@ -446,7 +498,11 @@ template <bool BWD, int AUXM>
 __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
-                                            uint32_t &n_con) {
+                                            uint32_t &n_con
+#ifdef DST_STATS
+                                            , WaveStats &ws
+#endif
+) {
     run.C[0] = run.C[1] = run.C[2] = 0.f;
     run.D = 0.f;
     run.N[0] = run.N[1] = run.N[2] = 0.f;
@@ -460,7 +516,15 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     while (__ballot(live) != 0ull) {
         kbuf_reset(buf);
         uint32_t cnt = 0;
+#ifdef DST_STATS
+        ws.chunks++;
+        unsigned long long c0 = __builtin_readcyclecounter();
+        packet_knn(acc, max_abs, ot, rd, live, buf, cnt, ws);
+        unsigned long long c1 = __builtin_readcyclecounter();
+        ws.t_trav += c1 - c0;
+#else
         packet_knn(acc, max_abs, ot, rd, live, buf, cnt);
+#endif
         int here = 0;
         bool stop = false;
         for (int it = 0; it < kChunk; ++it) {
@@ -468,13 +532,10 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             if (__ballot(on) == 0ull) break;
             // pop the front entry; the rest moves up (consumed slots need no reset: the buffer is
             // rebuilt from scratch for the next chunk)
-            const float e_t = buf.t[0];
-            const uint32_t e_i = buf.i[0];
+            const float e_t = kb_t(buf.e[0]);
+            const uint32_t e_i = kb_idx(buf.e[0]);
 #pragma unroll
-            for (int k = 0; k < kChunk - 1; ++k) {
-                buf.t[k] = buf.t[k + 1];
-                buf.i[k] = buf.i[k + 1];
-            }
+            for (int k = 0; k < kChunk - 1; ++k) buf.e[k] = buf.e[k + 1];
             if (!on) continue;
             const int g = (int)(e_i >> 1);
             if (g == last_g) continue;
@@ -545,6 +606,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
             Tp = Tn;
         }
+        STAT(ws.t_comp += __builtin_readcyclecounter() - c1;)
         if (live) {
             bool fin = (Tn < kTmin) || (cnt < (uint32_t)kChunk) || (contrib > kMaxContrib);
             const float next_dpt = (float)((double)dpt + kStepEps);
@@ -602,6 +664,12 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
     float *mid = p.mid_val + (size_t)slots * MID * r;
     const F3 ray_o = ld3(p.ray_o + 3 * r), ray_d = ld3(p.ray_d + 3 * r);
     uint32_t n_proc = 0, n_con = 0;
+#ifdef DST_STATS
+    WaveStats ws = {0, 0, 0, 0, 0, 0};
+#define WS_ARG , ws
+#else
+#define WS_ARG
+#endif
     BounceAcc<AUXM> run;
     BounceIn<AUXM> in;
     F3 g_ro = f3(0, 0, 0), g_rd = f3(0, 0, 0);
@@ -614,7 +682,7 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con);
+            walk_bounce<false, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -676,6 +744,14 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
             if (lane == 0) {
                 atomicAdd(p.counters + 0, (unsigned long long)a);
                 atomicAdd(p.counters + 1, (unsigned long long)b);
+#ifdef DST_STATS   // development build only: counters must then hold 8 entries
+                atomicAdd(p.counters + 2, ws.nodes);
+                atomicAdd(p.counters + 3, ws.leaves);
+                atomicAdd(p.counters + 4, ws.t_trav);
+                atomicAdd(p.counters + 5, ws.t_comp);
+                atomicAdd(p.counters + 6, ws.chunks);
+                atomicAdd(p.counters + 7, ws.leaf_any);
+#endif
             }
         }
     } else {
@@ -746,7 +822,7 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con);
+            walk_bounce<true, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con WS_ARG);
         }
         if (inside) {
             p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
@@ -780,11 +856,11 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     const uint64_t n_tiles64 = (uint64_t)tiles_x * tiles_y;
     if (n_tiles64 > 0x7FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
     DstAccelView acc;
-    acc.nodes = ctx->nodes;
+    acc.wide = ctx->wide;
     acc.leaves = ctx->leaves;
     acc.bounds = ctx->bounds;
     acc.n_leaves = ctx->n_leaves;
-    acc.root = (ctx->n_leaves == 1) ? (DST_LEAF_BIT | 0u) : 0u;
+    acc.root = dst_root_ref(ctx->n_leaves);
     if (backward)
         launch<true>(p, acc, tw_log2, th_log2, tiles_x, (uint32_t)n_tiles64, stream);
     else

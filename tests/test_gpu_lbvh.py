@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 LEAF = 0x80000000
 
 NODE = np.dtype([("lo0", "<f4", 3), ("hi0", "<f4", 3), ("lo1", "<f4", 3), ("hi1", "<f4", 3), ("c0", "<u4"),
-                 ("c1", "<u4"), ("pad", "<u4", 2)])
+                 ("c1", "<u4"), ("first", "<u4"), ("last", "<u4")])
 LEAFT = np.dtype([("A", "<f4", 3), ("B", "<f4", 3), ("C", "<f4", 3), ("D", "<f4", 3), ("g", "<u4"), ("pad", "<u4", 3)])
 
 
