@@ -326,6 +326,75 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
 
 __device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v); }
 
+// ---- per-block gradient table (backward) ---------------------------------------------------------------
+// The 16x16 pixel tile of a block keeps hitting the same few hundred surfels, so the per-surfel gradients
+// are first summed in an LDS hash table (one row of columns per surfel, LDS atomics) and written to
+// global memory once per surfel and block when the block ends.  A surfel that finds no free row within a
+// few probes goes straight to global atomics, so the table can never be wrong, only less effective.
+constexpr int kTableRows = 256;                 // power of two
+constexpr uint32_t kEmptyKey = 0xFFFFFFFFu;
+constexpr int kMaxProbe = 8;
+// row columns: colour 0-2, opacity 3, scales 4-5, rotation 6-9, mean 10-12, densification mean 13-15,
+// aux 16..16+AUXM-1, then SH coefficient j channel c at 16+AUXM+3j+c
+constexpr int kColColor = 0, kColOpac = 3, kColScale = 4, kColRot = 6, kColMean = 10, kColGrad = 13, kColAux = 16;
+template <int AUXM> struct RowLayout {
+    static constexpr int sh0 = kColAux + AUXM;
+    static constexpr int cols = sh0 + 48;
+    static constexpr int stride = cols | 1;     // odd: rows spread over all LDS banks
+};
+
+// Address in the caller's gradient tensors of column `col` of surfel g (nullptr: nothing to write).
+template <int AUXM>
+__device__ __forceinline__ float *grad_address(const DstParams &p, uint32_t g, int col) {
+    if (col < kColOpac) return p.dL_dcolors + 3 * (size_t)g + col;
+    if (col < kColScale) return p.dL_dopacities + g;
+    if (col < kColRot) return p.dL_dscales + 2 * (size_t)g + (col - kColScale);
+    if (col < kColMean) return p.dL_drotations + 4 * (size_t)g + (col - kColRot);
+    if (col < kColGrad) return p.dL_dmeans3D + 3 * (size_t)g + (col - kColMean);
+    if (col < kColAux) return p.dL_dgrads3D + 3 * (size_t)g + (col - kColGrad);
+    if (col < RowLayout<AUXM>::sh0) {
+        const int ch = col - kColAux;
+        return (p.others_precomp != nullptr && ch < p.aux) ? p.dL_dothers + (size_t)p.aux * g + ch : nullptr;
+    }
+    const int k = col - RowLayout<AUXM>::sh0;   // 3j + c
+    return (p.colors_precomp == nullptr && k < 3 * p.M) ? p.dL_dshs + (size_t)g * p.M * 3 + k : nullptr;
+}
+
+template <int AUXM>
+struct GradSink {
+    float *row;          // LDS row of this surfel, or nullptr: write through to global memory
+    const DstParams *p;
+    uint32_t g;
+    __device__ __forceinline__ void add(int col, float v) const {
+        if (row != nullptr) {
+            __hip_atomic_fetch_add(row + col, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+            float *dst = grad_address<AUXM>(*p, g, col);
+            if (dst != nullptr) aadd(dst, v);
+        }
+    }
+};
+
+// Find or claim the table row of surfel g.
+template <int AUXM>
+__device__ __forceinline__ float *table_row(uint32_t *keys, float *rows, uint32_t g) {
+    uint32_t slot = (g * 2654435761u) >> (32 - 8);
+    static_assert(kTableRows == 256, "hash shift assumes 256 rows");
+#pragma unroll 1
+    for (int probe = 0; probe < kMaxProbe; ++probe) {
+        uint32_t k = __hip_atomic_load(keys + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (k == kEmptyKey) {
+            uint32_t expected = kEmptyKey;
+            __hip_atomic_compare_exchange_strong(keys + slot, &expected, g, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_WORKGROUP);
+            k = (expected == kEmptyKey) ? g : expected;
+        }
+        if (k == g) return rows + (size_t)slot * RowLayout<AUXM>::stride;
+        slot = (slot + 1) & (kTableRows - 1);
+    }
+    return nullptr;
+}
+
 template <int AUXM>
 struct BounceIn {  // backward: saved results of the bounce and the gradients flowing into them
     float rgb[3], dpt, acc, nrm[3], aux[AUXM];
@@ -345,7 +414,8 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                                              F3 xyz, const F3 (&R)[3], float u, float v, float sx, float sy, F3 mean,
                                              float q0, float q1, float q2, float q3, float opac, float nsign,
                                              F3 normal, const float (&col)[3], const bool (&neg)[3], F3 ro, F3 rd,
-                                             const float *__restrict__ sh, F3 &g_ro, F3 &g_rd) {
+                                             const float *__restrict__ sh, F3 &g_ro, F3 &g_rd,
+                                             const GradSink<AUXM> &sink) {
 #pragma clang fp contract(fast)
     const float num = 1.0f - alpha;
     const float T_final = 1.0f - in.acc;
@@ -354,7 +424,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
 #pragma unroll
     for (int ch = 0; ch < 3; ++ch) {
         g_col[ch] = in.g_rgb[ch] * w;
-        aadd(p.dL_dcolors + 3 * (size_t)g + ch, g_col[ch]);
+        sink.add(kColColor + ch, g_col[ch]);
         g_alpha += in.g_rgb[ch] * (Tp * col[ch] - (in.rgb[ch] - run.C[ch]) / num);
         g_alpha += in.g_rgb[ch] * p.background[ch] * (-T_final / num);
     }
@@ -363,7 +433,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
         for (int ch = 0; ch < AUXM; ++ch) {
             if (ch < p.aux) {
                 float o = p.others_precomp[(size_t)p.aux * g + ch];
-                aadd(p.dL_dothers + (size_t)p.aux * g + ch, in.g_aux[ch] * w);
+                sink.add(kColAux + ch, in.g_aux[ch] * w);
                 g_alpha += in.g_aux[ch] * (Tp * o - (in.aux[ch] - run.O[ch]) / num);
             }
         }
@@ -377,7 +447,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     g_alpha += in.g_acc * (Tp - in.acc / num);   // the reference never accumulates W (backward.cu:568)
     const float g_G = g_alpha * opac;
     const float pc = (opac * G) > 0.99f ? 0.0f : 1.0f;
-    aadd(p.dL_dopacities + g, g_alpha * G * pc);
+    sink.add(kColOpac, g_alpha * G * pc);
 
     // triangle that was hit, with its corner coordinates in splat units (backward.cu:583-602)
     const float *V = p.vertices + (size_t)g * 12;
@@ -427,25 +497,22 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                           w_ * (gR[2].x - gR[0].z));
         float r3 = 2.f * (x * (gR[0].z + gR[2].x) + y * (gR[1].z + gR[2].y) - 2.f * z * (gR[0].x + gR[1].y) +
                           w_ * (gR[0].y - gR[1].x));
-        float *dr = p.dL_drotations + 4 * (size_t)g;
-        aadd(dr + 0, r0); aadd(dr + 1, r1); aadd(dr + 2, r2); aadd(dr + 3, r3);
+        sink.add(kColRot + 0, r0); sink.add(kColRot + 1, r1); sink.add(kColRot + 2, r2); sink.add(kColRot + 3, r3);
     }
-    aadd(p.dL_dscales + 2 * (size_t)g + 0, g_sx);
-    aadd(p.dL_dscales + 2 * (size_t)g + 1, g_sy);
-    float *dm = p.dL_dmeans3D + 3 * (size_t)g, *dg = p.dL_dgrads3D + 3 * (size_t)g;
-    aadd(dm + 0, g_mean.x); aadd(dm + 1, g_mean.y); aadd(dm + 2, g_mean.z);
+    sink.add(kColScale + 0, g_sx);
+    sink.add(kColScale + 1, g_sy);
+    sink.add(kColMean + 0, g_mean.x); sink.add(kColMean + 1, g_mean.y); sink.add(kColMean + 2, g_mean.z);
     const float hd = 0.5f * dpt;
-    aadd(dg + 0, g_mean.x * hd); aadd(dg + 1, g_mean.y * hd); aadd(dg + 2, g_mean.z * hd);
+    sink.add(kColGrad + 0, g_mean.x * hd); sink.add(kColGrad + 1, g_mean.y * hd); sink.add(kColGrad + 2, g_mean.z * hd);
 
     if (p.colors_precomp == nullptr) {
         // SH backward (backward.cu:68-166); the direction gradient REPLACES the ray's (backward.cu:165)
         const int deg = p.D;
         F3 gc = f3(neg[0] ? 0.f : g_col[0], neg[1] ? 0.f : g_col[1], neg[2] ? 0.f : g_col[2]);
-        float *ds = p.dL_dshs + (size_t)g * p.M * 3;
         auto put = [&](int j, float basis) {
-            aadd(ds + 3 * j + 0, basis * gc.x);
-            aadd(ds + 3 * j + 1, basis * gc.y);
-            aadd(ds + 3 * j + 2, basis * gc.z);
+            sink.add(RowLayout<AUXM>::sh0 + 3 * j + 0, basis * gc.x);
+            sink.add(RowLayout<AUXM>::sh0 + 3 * j + 1, basis * gc.y);
+            sink.add(RowLayout<AUXM>::sh0 + 3 * j + 2, basis * gc.z);
         };
         auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
         F3 ddx = f3(0, 0, 0), ddy = f3(0, 0, 0), ddz = f3(0, 0, 0);
@@ -498,7 +565,7 @@ template <bool BWD, int AUXM>
 __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
-                                            uint32_t &n_con
+                                            uint32_t &n_con, uint32_t *tab_keys, float *tab_rows
 #ifdef DST_STATS
                                             , WaveStats &ws
 #endif
@@ -599,8 +666,12 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             n_con++;
             here++;
             if (BWD) {
+                GradSink<AUXM> sink;
+                sink.row = table_row<AUXM>(tab_keys, tab_rows, (uint32_t)g);
+                sink.p = &p;
+                sink.g = (uint32_t)g;
                 hit_backward<AUXM>(p, in, run, g, e_i, Tp, alpha, G, w, dpt, xyz, R, u, v, sx, sy, mean, q0, q1, q2, q3,
-                                   opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd);
+                                   opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink);
             } else if (p.training && p.a_weights != nullptr) {
                 aadd(p.a_weights + g, w);
             }
@@ -649,14 +720,27 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
 template <bool BWD, int AUXM>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstParams p, const DstAccelView acc,
                                                                      int tw_log2, int th_log2, uint32_t tiles_x,
-                                                                     uint32_t n_tiles) {
-    const uint32_t tile = blockIdx.x * kWavesPerBlock + (threadIdx.x / DST_WAVE);
-    if (tile >= n_tiles) return;
+                                                                     uint32_t tiles_y, uint32_t btiles_x) {
+    // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
+    // is what the block's gradient table and the caches live on
+    __shared__ uint32_t s_keys[BWD ? kTableRows : 1];
+    __shared__ float s_rows[BWD ? kTableRows * RowLayout<AUXM>::stride : 1];
+    uint32_t *tab_keys = s_keys;
+    float *tab_rows = s_rows;
+    if (BWD) {
+        for (int k = threadIdx.x; k < kTableRows; k += kWavesPerBlock * DST_WAVE) s_keys[k] = kEmptyKey;
+        for (int k = threadIdx.x; k < kTableRows * RowLayout<AUXM>::stride; k += kWavesPerBlock * DST_WAVE)
+            s_rows[k] = 0.f;
+        __syncthreads();
+    }
+    const uint32_t wv = threadIdx.x / DST_WAVE;
+    const uint32_t ty = 2u * (blockIdx.x / btiles_x) + (wv >> 1), tx = 2u * (blockIdx.x % btiles_x) + (wv & 1u);
+    const bool wave_on = ty < tiles_y && tx < tiles_x;
+    if (!BWD && !wave_on) return;   // the backward kernel keeps every wave for the block-wide flush below
     const uint32_t lane = threadIdx.x % DST_WAVE;
-    const uint32_t ty = tile / tiles_x, tx = tile % tiles_x;
     const uint32_t py = (ty << th_log2) + (lane >> tw_log2);
     const uint32_t px = (tx << tw_log2) + (lane & ((1u << tw_log2) - 1u));
-    const bool inside = py < (uint32_t)p.H && px < (uint32_t)p.W;
+    const bool inside = wave_on && py < (uint32_t)p.H && px < (uint32_t)p.W;
     const size_t r = inside ? ((size_t)py * p.W + px) : 0;
     const float max_abs = __uint_as_float(acc.bounds->max_abs);
     const int MID = 14 + p.aux, AUXO = 11, RGBO = 11 + p.aux;
@@ -682,7 +766,7 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con WS_ARG);
+            walk_bounce<false, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -822,25 +906,39 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con WS_ARG);
+            walk_bounce<true, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows WS_ARG);
         }
         if (inside) {
             p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
             p.dL_dray_d[3 * r + 0] = g_rd.x; p.dL_dray_d[3 * r + 1] = g_rd.y; p.dL_dray_d[3 * r + 2] = g_rd.z;
         }
+        // flush the block's table: consecutive threads take consecutive columns of a row, so the 48 SH
+        // columns of a surfel go out as contiguous atomics
+        __syncthreads();
+        constexpr int stride = RowLayout<AUXM>::stride;
+        for (int k = threadIdx.x; k < kTableRows * stride; k += kWavesPerBlock * DST_WAVE) {
+            const int row = k / stride, col = k - row * stride;
+            const uint32_t g = s_keys[row];
+            if (g == kEmptyKey || col >= RowLayout<AUXM>::cols) continue;
+            const float v = s_rows[k];
+            if (v == 0.f) continue;
+            float *dst = grad_address<AUXM>(p, g, col);
+            if (dst != nullptr) aadd(dst, v);
+        }
     }
 }
 
 template <bool BWD>
-void launch(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2, uint32_t tiles_x, uint32_t n_tiles,
+void launch(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2, uint32_t tiles_x, uint32_t tiles_y,
             hipStream_t stream) {
-    dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock), block(kWavesPerBlock * DST_WAVE);
+    const uint32_t btiles_x = (tiles_x + 1) / 2, btiles_y = (tiles_y + 1) / 2;
+    dim3 grid(btiles_x * btiles_y), block(kWavesPerBlock * DST_WAVE);
     if (p.aux <= 2)
-        hipLaunchKernelGGL((k_trace<BWD, 2>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, n_tiles);
+        hipLaunchKernelGGL((k_trace<BWD, 2>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
     else if (p.aux <= 4)
-        hipLaunchKernelGGL((k_trace<BWD, 4>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, n_tiles);
+        hipLaunchKernelGGL((k_trace<BWD, 4>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
     else
-        hipLaunchKernelGGL((k_trace<BWD, 8>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, n_tiles);
+        hipLaunchKernelGGL((k_trace<BWD, 8>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
 }
 
 }  // namespace
@@ -853,8 +951,7 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     const int tw_log2 = 6 - th_log2;
     const uint32_t tiles_x = ((uint32_t)p.W + (1u << tw_log2) - 1) >> tw_log2;
     const uint32_t tiles_y = ((uint32_t)p.H + (1u << th_log2) - 1) >> th_log2;
-    const uint64_t n_tiles64 = (uint64_t)tiles_x * tiles_y;
-    if (n_tiles64 > 0x7FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
+    if ((uint64_t)tiles_x * tiles_y > 0x7FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
     DstAccelView acc;
     acc.wide = ctx->wide;
     acc.leaves = ctx->leaves;
@@ -862,9 +959,9 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     acc.n_leaves = ctx->n_leaves;
     acc.root = dst_root_ref(ctx->n_leaves);
     if (backward)
-        launch<true>(p, acc, tw_log2, th_log2, tiles_x, (uint32_t)n_tiles64, stream);
+        launch<true>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, stream);
     else
-        launch<false>(p, acc, tw_log2, th_log2, tiles_x, (uint32_t)n_tiles64, stream);
+        launch<false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, stream);
     DST_HIP(ctx, hipGetLastError());
     return DST_OK;
 }
