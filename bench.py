@@ -95,10 +95,12 @@ def main():
     counters = torch.zeros(2, dtype=torch.int64, device=dev)
 
     def step(fwd_events=None, bwd_events=None, count=False):
+        # what the autograd function does: the forward trace records its hit buffers, backward replays them
+        rec = _C.HitRecord(H, W, 1, ctx.record_blocks_per_wave, dev)
         out = _C.trace_surfels(ctx, True, True, ro, rd, *common, counters=counters if count else None,
-                               events=fwd_events)
+                               events=fwd_events, hit_record=rec)
         grads = _C.trace_surfels_backward(ctx, True, ro, rd, *common, *out[:7], ug["rgb"], ug["dpt"], ug["acc"],
-                                          ug["norm"], ug["dist"], ug["aux"], events=bwd_events)
+                                          ug["norm"], ug["dist"], ug["aux"], events=bwd_events, hit_record=rec)
         return out, grads
 
     for _ in range(args.warmup):
@@ -124,8 +126,8 @@ def main():
     A_total = A_fwd + A_bwd + PER_SURFEL_INIT * P
     rays_per_s = R / (ms_per_step * 1e-3)
 
-    dominant = ("backward", "k_trace<true,2>", A_bwd, bwd_ms) if bwd_ms >= fwd_ms else \
-        ("forward", "k_trace<false,2>", A_fwd, fwd_ms)
+    dominant = ("backward", "k_trace<true,2,true>", A_bwd, bwd_ms) if bwd_ms >= fwd_ms else \
+        ("forward", "k_trace<false,2,true>", A_fwd, fwd_ms)
     achieved = dominant[2] / (dominant[3] * 1e-3) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")

@@ -32,6 +32,8 @@ int check_common(dst_ctx *ctx, const DstParams *p) {
     if (!p->vertices || !p->background || !p->means3D || !p->opacities || !p->scales || !p->rotations)
         return dst_fail(ctx, DST_E_INVALID,
                         "vertices, background, means3D, opacities, scales and rotations are required");
+    if (p->hit_record && (reinterpret_cast<uintptr_t>(p->hit_record) & 7u))
+        return dst_fail(ctx, DST_E_INVALID, "hit_record must be 8-byte aligned");
     if (p->H > 0 && p->W > 0 &&
         (!p->out_rgb || !p->out_dpt || !p->out_acc || !p->out_norm || !p->out_dist || !p->out_aux || !p->mid_val))
         return dst_fail(ctx, DST_E_INVALID, "forward output buffers missing");

@@ -360,17 +360,74 @@ __device__ __forceinline__ float *grad_address(const DstParams &p, uint32_t g, i
     return (p.colors_precomp == nullptr && k < 3 * p.M) ? p.dL_dshs + (size_t)g * p.M * 3 + k : nullptr;
 }
 
+// Sum of v over the 64 lanes; every lane must be active.
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#define DST_DPP_ADD(ctrl, rmask)                                                                              \
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xf, true))
+    DST_DPP_ADD(0x111, 0xf);   // row_shr:1
+    DST_DPP_ADD(0x112, 0xf);   // row_shr:2
+    DST_DPP_ADD(0x114, 0xf);   // row_shr:4
+    DST_DPP_ADD(0x118, 0xf);   // row_shr:8   -> lane 15 of each row holds the row total
+    DST_DPP_ADD(0x142, 0xa);   // row_bcast:15 into rows 1 and 3
+    DST_DPP_ADD(0x143, 0xc);   // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave total
+#undef DST_DPP_ADD
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));   // the builtin moves bits of an int
+}
+
+// Where one hit's per-surfel gradients go.  Lanes of a wave that composite the SAME surfel in the same step
+// would serialise on the same LDS addresses, so the largest groups of such lanes (found once per step) are
+// summed across the wave first and only their first lane issues the atomic; all other lanes add directly.
+constexpr int kBigGroups = 3;       // groups reduced across the wave per step
+constexpr int kBigGroupMin = 8;     // lanes a group needs before the reduction pays
 template <int AUXM>
 struct GradSink {
-    float *row;          // LDS row of this surfel, or nullptr: write through to global memory
+    float *row;          // LDS row of this lane's surfel, or nullptr: write through to global memory
     const DstParams *p;
     uint32_t g;
+    int n_big;           // wave-uniform
+    int member;          // index of the big group this lane belongs to, or -1
+    bool lead;           // this lane issues the atomic of its big group
+    bool direct;         // this lane adds its own value (not in a big group)
+
+    // Wave-uniform: `key` is the surfel of lanes with a hit, anything for the others.
+    __device__ __forceinline__ void plan(bool did, uint32_t key) {
+        const uint32_t lane = __lane_id();
+        uint64_t rem = __ballot(did);
+        n_big = 0;
+        member = -1;
+        lead = false;
+        for (int tries = 0; tries < 2 * kBigGroups && rem != 0ull && n_big < kBigGroups; ++tries) {
+            const int first = __builtin_ctzll(rem);
+            const uint32_t k0 = __builtin_amdgcn_readlane(key, first);
+            const bool same = did && key == k0;
+            const uint64_t grp = __ballot(same);
+            if (__popcll(grp) >= kBigGroupMin) {
+                if (same) member = n_big;
+                if (lane == (uint32_t)first) lead = true;
+                ++n_big;
+            }
+            rem &= ~grp;
+        }
+        direct = did && member < 0;
+    }
+
+    // Wave-uniform call (every lane reaches it); lanes without a hit contribute nothing.
     __device__ __forceinline__ void add(int col, float v) const {
-        if (row != nullptr) {
-            __hip_atomic_fetch_add(row + col, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        } else {
-            float *dst = grad_address<AUXM>(*p, g, col);
-            if (dst != nullptr) aadd(dst, v);
+        float out = v;
+#pragma unroll
+        for (int k = 0; k < kBigGroups; ++k) {
+            if (k < n_big) {
+                const float s = wave_sum_f32(member == k ? v : 0.f);
+                out = (member == k) ? s : out;
+            }
+        }
+        if (direct || lead) {
+            if (row != nullptr) {
+                __hip_atomic_fetch_add(row + col, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+                float *dst = grad_address<AUXM>(*p, g, col);
+                if (dst != nullptr) aadd(dst, out);
+            }
         }
     }
 };
@@ -415,7 +472,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                                              float q0, float q1, float q2, float q3, float opac, float nsign,
                                              F3 normal, const float (&col)[3], const bool (&neg)[3], F3 ro, F3 rd,
                                              const float *__restrict__ sh, F3 &g_ro, F3 &g_rd,
-                                             const GradSink<AUXM> &sink) {
+                                             const GradSink<AUXM> &sink, bool did) {
 #pragma clang fp contract(fast)
     const float num = 1.0f - alpha;
     const float T_final = 1.0f - in.acc;
@@ -477,8 +534,10 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     const F3 g_v1 = g_d * cross(v2 - v3, g_n) + g_d * n / q;
     const F3 g_v2 = g_d * cross(v3 - v1, g_n);
     const F3 g_v3 = g_d * cross(v1 - v2, g_n);
-    g_ro = g_ro + (g_xyz + (g_d * -n) / q);
-    g_rd = g_rd + (g_xyz * dpt + ((g_d * -pp) / (q * q)) * n);
+    if (did) {
+        g_ro = g_ro + (g_xyz + (g_d * -n) / q);
+        g_rd = g_rd + (g_xyz * dpt + ((g_d * -pp) / (q * q)) * n);
+    }
     const F3 su = h1.x * g_v1 + h2.x * g_v2 + h3.x * g_v3;
     const F3 sv = h1.y * g_v1 + h2.y * g_v2 + h3.y * g_v3;
     gR[0] = gR[0] + sx * su;
@@ -555,17 +614,65 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                 }
             }
         }
-        g_rd = f3(dot(ddx, gc), dot(ddy, gc), dot(ddz, gc));
+        if (did) g_rd = f3(dot(ddx, gc), dot(ddy, gc), dot(ddz, gc));
     }
+}
+
+// ---- hit record: the forward trace can store every chunk's hit buffer, the backward trace then replays
+// them instead of walking the BVH again.  Layout of the caller's buffer, in 8-byte words:
+//   [0] blocks requested so far (the forward kernel counts on past the capacity, which is how overflow shows)
+//   [1] unused
+//   [2 ...) directory: one uint32 per (wave, bounce slot) = 1 + first block of that wave's bounce, 0 = none
+//   then `capacity` blocks of kRecBlockWords words: 16x64 entries ([slot][lane]), 64 uint32 counts, next+1.
+constexpr uint32_t kRecBlockWords = kChunk * DST_WAVE + DST_WAVE / 2 + 8;
+struct RecView {
+    uint64_t *base;      // nullptr: not recording / not replaying
+    uint64_t *blocks;    // first block
+    uint32_t *dir;       // this wave's directory entries (one per bounce slot)
+    uint32_t capacity;
+};
+
+// Forward: append one chunk of this wave to the record.  `prev` is the wave's previous block in this bounce.
+__device__ __forceinline__ void rec_store(const RecView &rv, int bounce, uint32_t &prev, const KBuf &buf, uint32_t cnt) {
+    const uint32_t lane = __lane_id();
+    uint32_t blk = 0;
+    if (lane == 0) blk = (uint32_t)atomicAdd((unsigned long long *)rv.base, 1ull);
+    blk = __builtin_amdgcn_readfirstlane(blk);
+    if (blk >= rv.capacity) return;   // too small: the host sees the count and the backward pass re-traces
+    uint64_t *b = rv.blocks + (size_t)blk * kRecBlockWords;
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) b[k * DST_WAVE + lane] = buf.e[k];
+    uint32_t *cnts = reinterpret_cast<uint32_t *>(b + kChunk * DST_WAVE);
+    cnts[lane] = cnt;
+    if (lane == 0) {
+        cnts[DST_WAVE] = 0u;   // next: none yet
+        if (prev == 0xFFFFFFFFu) rv.dir[bounce] = blk + 1u;
+        else reinterpret_cast<uint32_t *>(rv.blocks + (size_t)prev * kRecBlockWords + kChunk * DST_WAVE)[DST_WAVE] = blk + 1u;
+    }
+    prev = blk;
+}
+
+// Backward: fetch the next chunk of this wave's bounce.  Returns false when the chain ends early.
+__device__ __forceinline__ bool rec_load(const RecView &rv, uint32_t &cur, KBuf &buf, uint32_t &cnt) {
+    if (cur == 0u || cur > rv.capacity) return false;
+    const uint32_t lane = __lane_id();
+    const uint64_t *b = rv.blocks + (size_t)(cur - 1u) * kRecBlockWords;
+#pragma unroll
+    for (int k = 0; k < kChunk; ++k) buf.e[k] = b[k * DST_WAVE + lane];
+    const uint32_t *cnts = reinterpret_cast<const uint32_t *>(b + kChunk * DST_WAVE);
+    cnt = cnts[lane];
+    cur = __builtin_amdgcn_readfirstlane(cnts[DST_WAVE]);
+    return true;
 }
 
 // One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
 // and for BWD the per-hit gradients of the re-trace (reference backward.cu:332-655).
-template <bool BWD, int AUXM>
+template <bool BWD, int AUXM, bool REC>
 __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
-                                            uint32_t &n_con, uint32_t *tab_keys, float *tab_rows
+                                            uint32_t &n_con, uint32_t *tab_keys, float *tab_rows, const RecView &rv,
+                                            int bounce
 #ifdef DST_STATS
                                             , WaveStats &ws
 #endif
@@ -580,18 +687,18 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     F3 ot = ro;
     bool live = lane_on;
     KBuf buf;
+    uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
     while (__ballot(live) != 0ull) {
-        kbuf_reset(buf);
         uint32_t cnt = 0;
-#ifdef DST_STATS
-        ws.chunks++;
-        unsigned long long c0 = __builtin_readcyclecounter();
-        packet_knn(acc, max_abs, ot, rd, live, buf, cnt, ws);
-        unsigned long long c1 = __builtin_readcyclecounter();
-        ws.t_trav += c1 - c0;
-#else
-        packet_knn(acc, max_abs, ot, rd, live, buf, cnt);
-#endif
+        STAT(ws.chunks++; unsigned long long c0 = __builtin_readcyclecounter();)
+        if (REC && BWD) {
+            if (!rec_load(rv, rec_pos, buf, cnt)) break;   // cannot happen with a complete record
+        } else {
+            kbuf_reset(buf);
+            packet_knn(acc, max_abs, ot, rd, live, buf, cnt WSP);
+            if (REC && !BWD) rec_store(rv, bounce, rec_pos, buf, cnt);
+        }
+        STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
         int here = 0;
         bool stop = false;
         for (int it = 0; it < kChunk; ++it) {
@@ -603,79 +710,93 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             const uint32_t e_i = kb_idx(buf.e[0]);
 #pragma unroll
             for (int k = 0; k < kChunk - 1; ++k) buf.e[k] = buf.e[k + 1];
-            if (!on) continue;
-            const int g = (int)(e_i >> 1);
-            if (g == last_g) continue;
-            dpt = e_t + pay_dpt;
-            const F3 xyz = f3(ro.x + dpt * rd.x, ro.y + dpt * rd.y, ro.z + dpt * rd.z);
-            const F3 mean = ld3(p.means3D + 3 * (size_t)g);
-            const float sx = p.scales[2 * (size_t)g], sy = p.scales[2 * (size_t)g + 1];
-            const float *qp = p.rotations + 4 * (size_t)g;
-            const float q0 = qp[0], q1 = qp[1], q2 = qp[2], q3 = qp[3];
-            F3 R[3];
-            quat_rows(q0, q1, q2, q3, R);
-            const float Tx = dot(R[0], mean), Ty = dot(R[1], mean);
-            const float ux = R[0].x * xyz.x + R[0].y * xyz.y + R[0].z * xyz.z + (-Tx);
-            const float uy = R[1].x * xyz.x + R[1].y * xyz.y + R[1].z * xyz.z + (-Ty);
-            const float u = ux / sx, v = uy / sy;
-            const float rho = u * u + v * v;
-            n_proc++;
-            F3 normal = R[2];
-            const float cosv = -(rd.x * normal.x + rd.y * normal.y + rd.z * normal.z);
-            if (cosv == 0.f) continue;
-            const float nsign = cosv > 0.f ? 1.0f : -1.0f;
-            normal = cosv > 0.f ? normal : -normal;
-            if (dpt < min_depth) continue;
-            const float power = -0.5f * rho;
-            if (power > 0.0f) continue;
-            const float opac = p.opacities[g];
-            const float G = exp_det(power);
-            float alpha = opac * G;
-            alpha = (alpha < 0.99f) ? alpha : 0.99f;
-            if (alpha < 1.0f / 255.0f) continue;
-            Tn = Tp * (1 - alpha);
-            if (Tn < kTmin) { stop = true; continue; }
-            contrib++;
-            if (contrib > kMaxContrib) { stop = true; continue; }
-            last_g = g;
-            const float w = alpha * Tp;
-            float col[3];
+            // ---- phase 1 (per lane): evaluate the entry, decide, composite ------------------------------
+            bool did = false;          // this lane composited a hit in this iteration
+            int g = 0;
+            float Tp_hit = 1.f, alpha = 0.f, G = 0.f, w = 0.f, u = 0.f, v = 0.f, sx = 1.f, sy = 1.f, opac = 0.f;
+            float nsign = 1.f, q0 = 1.f, q1 = 0.f, q2 = 0.f, q3 = 0.f, dpt_hit = 0.f;
+            F3 xyz = f3(0, 0, 0), mean = f3(0, 0, 0), normal = f3(0, 0, 1);
+            F3 R[3] = {f3(1, 0, 0), f3(0, 1, 0), f3(0, 0, 1)};
+            float col[3] = {0.f, 0.f, 0.f};
             bool neg[3] = {false, false, false};
-            const float *sh = nullptr;
-            if (p.colors_precomp == nullptr) {
-                sh = p.shs + (size_t)g * p.M * 3;
-                F3 c = sh_color(p.D, sh, rd, neg);
-                col[0] = c.x; col[1] = c.y; col[2] = c.z;
-            } else {
-                col[0] = p.colors_precomp[3 * (size_t)g];
-                col[1] = p.colors_precomp[3 * (size_t)g + 1];
-                col[2] = p.colors_precomp[3 * (size_t)g + 2];
-            }
-            run.C[0] += w * col[0];
-            run.C[1] += w * col[1];
-            run.C[2] += w * col[2];
-            if (p.others_precomp != nullptr) {
+            const float *sh = p.shs;   // valid address for lanes that sit phase 2 out
+            do {
+                if (!on) break;
+                g = (int)(e_i >> 1);
+                if (g == last_g) break;
+                dpt = e_t + pay_dpt;
+                xyz = f3(ro.x + dpt * rd.x, ro.y + dpt * rd.y, ro.z + dpt * rd.z);
+                mean = ld3(p.means3D + 3 * (size_t)g);
+                sx = p.scales[2 * (size_t)g];
+                sy = p.scales[2 * (size_t)g + 1];
+                const float *qp = p.rotations + 4 * (size_t)g;
+                q0 = qp[0]; q1 = qp[1]; q2 = qp[2]; q3 = qp[3];
+                quat_rows(q0, q1, q2, q3, R);
+                const float Tx = dot(R[0], mean), Ty = dot(R[1], mean);
+                const float ux = R[0].x * xyz.x + R[0].y * xyz.y + R[0].z * xyz.z + (-Tx);
+                const float uy = R[1].x * xyz.x + R[1].y * xyz.y + R[1].z * xyz.z + (-Ty);
+                u = ux / sx;
+                v = uy / sy;
+                const float rho = u * u + v * v;
+                n_proc++;
+                normal = R[2];
+                const float cosv = -(rd.x * normal.x + rd.y * normal.y + rd.z * normal.z);
+                if (cosv == 0.f) break;
+                nsign = cosv > 0.f ? 1.0f : -1.0f;
+                normal = cosv > 0.f ? normal : -normal;
+                if (dpt < min_depth) break;
+                const float power = -0.5f * rho;
+                if (power > 0.0f) break;
+                opac = p.opacities[g];
+                G = exp_det(power);
+                alpha = opac * G;
+                alpha = (alpha < 0.99f) ? alpha : 0.99f;
+                if (alpha < 1.0f / 255.0f) break;
+                Tn = Tp * (1 - alpha);
+                if (Tn < kTmin) { stop = true; break; }
+                contrib++;
+                if (contrib > kMaxContrib) { stop = true; break; }
+                last_g = g;
+                w = alpha * Tp;
+                if (p.colors_precomp == nullptr) {
+                    sh = p.shs + (size_t)g * p.M * 3;
+                    F3 c = sh_color(p.D, sh, rd, neg);
+                    col[0] = c.x; col[1] = c.y; col[2] = c.z;
+                } else {
+                    col[0] = p.colors_precomp[3 * (size_t)g];
+                    col[1] = p.colors_precomp[3 * (size_t)g + 1];
+                    col[2] = p.colors_precomp[3 * (size_t)g + 2];
+                }
+                run.C[0] += w * col[0];
+                run.C[1] += w * col[1];
+                run.C[2] += w * col[2];
+                if (p.others_precomp != nullptr) {
 #pragma unroll
-                for (int ch = 0; ch < AUXM; ++ch)
-                    if (ch < p.aux) run.O[ch] += w * p.others_precomp[(size_t)p.aux * g + ch];
-            }
-            run.D += w * dpt;
-            run.N[0] += w * normal.x;
-            run.N[1] += w * normal.y;
-            run.N[2] += w * normal.z;
-            n_con++;
-            here++;
-            if (BWD) {
+                    for (int ch = 0; ch < AUXM; ++ch)
+                        if (ch < p.aux) run.O[ch] += w * p.others_precomp[(size_t)p.aux * g + ch];
+                }
+                run.D += w * dpt;
+                run.N[0] += w * normal.x;
+                run.N[1] += w * normal.y;
+                run.N[2] += w * normal.z;
+                n_con++;
+                here++;
+                did = true;
+                Tp_hit = Tp;
+                dpt_hit = dpt;
+                Tp = Tn;
+                if (!BWD && p.training && p.a_weights != nullptr) aadd(p.a_weights + g, w);
+            } while (false);
+            // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
+            if (BWD && __ballot(did) != 0ull) {
                 GradSink<AUXM> sink;
-                sink.row = table_row<AUXM>(tab_keys, tab_rows, (uint32_t)g);
+                sink.plan(did, did ? (uint32_t)g : 0xFFFFFFFFu);
+                sink.row = did ? table_row<AUXM>(tab_keys, tab_rows, (uint32_t)g) : nullptr;
                 sink.p = &p;
                 sink.g = (uint32_t)g;
-                hit_backward<AUXM>(p, in, run, g, e_i, Tp, alpha, G, w, dpt, xyz, R, u, v, sx, sy, mean, q0, q1, q2, q3,
-                                   opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink);
-            } else if (p.training && p.a_weights != nullptr) {
-                aadd(p.a_weights + g, w);
+                hit_backward<AUXM>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
+                                   q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did);
             }
-            Tp = Tn;
         }
         STAT(ws.t_comp += __builtin_readcyclecounter() - c1;)
         if (live) {
@@ -717,7 +838,7 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
     return v;
 }
 
-template <bool BWD, int AUXM>
+template <bool BWD, int AUXM, bool REC>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstParams p, const DstAccelView acc,
                                                                      int tw_log2, int th_log2, uint32_t tiles_x,
                                                                      uint32_t tiles_y, uint32_t btiles_x) {
@@ -734,6 +855,15 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
         __syncthreads();
     }
     const uint32_t wv = threadIdx.x / DST_WAVE;
+    RecView rv = {nullptr, nullptr, nullptr, 0u};
+    if (REC) {
+        const uint32_t n_waves = gridDim.x * kWavesPerBlock, slots_ = (uint32_t)p.mtd_alloc + 1u;
+        const uint64_t dir_words = ((uint64_t)n_waves * slots_ + 1u) / 2u;
+        rv.base = p.hit_record;
+        rv.dir = reinterpret_cast<uint32_t *>(p.hit_record + 2) + (size_t)(blockIdx.x * kWavesPerBlock + wv) * slots_;
+        rv.blocks = p.hit_record + 2 + dir_words;
+        rv.capacity = p.hit_record_blocks;
+    }
     const uint32_t ty = 2u * (blockIdx.x / btiles_x) + (wv >> 1), tx = 2u * (blockIdx.x % btiles_x) + (wv & 1u);
     const bool wave_on = ty < tiles_y && tx < tiles_x;
     if (!BWD && !wave_on) return;   // the backward kernel keeps every wave for the block-wide flush below
@@ -766,7 +896,7 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr WS_ARG);
+            walk_bounce<false, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, rv, i WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -906,7 +1036,7 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows WS_ARG);
+            walk_bounce<true, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, rv, i WS_ARG);
         }
         if (inside) {
             p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
@@ -928,40 +1058,73 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
     }
 }
 
-template <bool BWD>
-void launch(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2, uint32_t tiles_x, uint32_t tiles_y,
-            hipStream_t stream) {
-    const uint32_t btiles_x = (tiles_x + 1) / 2, btiles_y = (tiles_y + 1) / 2;
-    dim3 grid(btiles_x * btiles_y), block(kWavesPerBlock * DST_WAVE);
+struct TileGrid {
+    int tw_log2, th_log2;
+    uint32_t tiles_x, tiles_y, btiles_x, btiles_y;
+};
+
+// 8x8 pixel tiles per wave, 2x2 tiles per block; thin grids (H < 8, e.g. (1,N,3) ray lists) get wider, flatter tiles.
+TileGrid tile_grid(int H, int W) {
+    TileGrid t;
+    t.th_log2 = 3;
+    while (t.th_log2 > 0 && (1 << t.th_log2) > H) --t.th_log2;
+    t.tw_log2 = 6 - t.th_log2;
+    t.tiles_x = ((uint32_t)W + (1u << t.tw_log2) - 1) >> t.tw_log2;
+    t.tiles_y = ((uint32_t)H + (1u << t.th_log2) - 1) >> t.th_log2;
+    t.btiles_x = (t.tiles_x + 1) / 2;
+    t.btiles_y = (t.tiles_y + 1) / 2;
+    return t;
+}
+
+template <bool BWD, bool REC>
+void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipStream_t stream) {
+    dim3 grid(t.btiles_x * t.btiles_y), block(kWavesPerBlock * DST_WAVE);
     if (p.aux <= 2)
-        hipLaunchKernelGGL((k_trace<BWD, 2>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+        hipLaunchKernelGGL((k_trace<BWD, 2, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2, t.tiles_x,
+                           t.tiles_y, t.btiles_x);
     else if (p.aux <= 4)
-        hipLaunchKernelGGL((k_trace<BWD, 4>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+        hipLaunchKernelGGL((k_trace<BWD, 4, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2, t.tiles_x,
+                           t.tiles_y, t.btiles_x);
     else
-        hipLaunchKernelGGL((k_trace<BWD, 8>), grid, block, 0, stream, p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+        hipLaunchKernelGGL((k_trace<BWD, 8, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2, t.tiles_x,
+                           t.tiles_y, t.btiles_x);
 }
 
 }  // namespace
 
+uint64_t dst_hit_record_layout(int32_t H, int32_t W, int32_t mtd_alloc, uint32_t blocks, uint64_t *header_words,
+                               uint32_t *n_waves) {
+    if (H <= 0 || W <= 0 || mtd_alloc < 0) {
+        if (header_words) *header_words = 0;
+        if (n_waves) *n_waves = 0;
+        return 0;
+    }
+    const TileGrid t = tile_grid(H, W);
+    const uint64_t waves = (uint64_t)t.btiles_x * t.btiles_y * kWavesPerBlock;
+    const uint64_t header = 2 + (waves * (uint64_t)(mtd_alloc + 1) + 1) / 2;
+    if (header_words) *header_words = header;
+    if (n_waves) *n_waves = (uint32_t)waves;
+    return header + (uint64_t)blocks * kRecBlockWords;
+}
+
 int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream) {
     if (p.H <= 0 || p.W <= 0) return DST_OK;  // empty ray grid: nothing to do
-    // 8x8 pixel tiles per wave; thin grids (H < 8, e.g. (1,N,3) ray lists) get wider, flatter tiles
-    int th_log2 = 3;
-    while (th_log2 > 0 && (1 << th_log2) > p.H) --th_log2;
-    const int tw_log2 = 6 - th_log2;
-    const uint32_t tiles_x = ((uint32_t)p.W + (1u << tw_log2) - 1) >> tw_log2;
-    const uint32_t tiles_y = ((uint32_t)p.H + (1u << th_log2) - 1) >> th_log2;
-    if ((uint64_t)tiles_x * tiles_y > 0x7FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
+    const TileGrid t = tile_grid(p.H, p.W);
+    if ((uint64_t)t.tiles_x * t.tiles_y > 0x3FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
     DstAccelView acc;
     acc.wide = ctx->wide;
     acc.leaves = ctx->leaves;
     acc.bounds = ctx->bounds;
     acc.n_leaves = ctx->n_leaves;
     acc.root = dst_root_ref(ctx->n_leaves);
-    if (backward)
-        launch<true>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, stream);
-    else
-        launch<false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, stream);
+    const bool rec = p.hit_record != nullptr;
+    if (backward) {
+        if (rec) launch<true, true>(p, acc, t, stream);
+        else launch<true, false>(p, acc, t, stream);
+    } else {
+        if (rec) launch<false, true>(p, acc, t, stream);
+        else launch<false, false>(p, acc, t, stream);
+    }
     DST_HIP(ctx, hipGetLastError());
     return DST_OK;
 }

@@ -29,7 +29,8 @@ class DstParams(C.Structure):
         + [(n, _FP) for n in ("ray_o", "ray_d", "vertices", "background", "means3D", "shs", "colors_precomp",
                               "others_precomp", "opacities", "scales", "rotations")]
         + [(n, _FP) for n in ("out_rgb", "out_dpt", "out_acc", "out_norm", "out_dist", "out_aux", "mid_val",
-                              "a_weights", "counters")]
+                              "a_weights", "counters", "hit_record")]
+        + [("hit_record_blocks", C.c_uint32), ("reserved0", C.c_uint32)]
         + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
         + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
                               "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
@@ -43,7 +44,8 @@ class DstAccelInfo(C.Structure):
 
 
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
-           "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params")
+           "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params",
+           "dst_hit_record_layout")
 
 _lib = None
 
@@ -70,6 +72,9 @@ def load_library():
     L.dst_accel_download.argtypes = [C.c_void_p] * 7
     L.dst_version.restype = C.c_char_p
     L.dst_sizeof_params.restype = C.c_size_t
+    L.dst_hit_record_layout.restype = C.c_uint64
+    L.dst_hit_record_layout.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_uint32, C.POINTER(C.c_uint64),
+                                        C.POINTER(C.c_uint32)]
     if L.dst_sizeof_params() != C.sizeof(DstParams):
         raise ImportError("diff_surfel_tracing: DstParams layout mismatch between _C.py and libdst.so")
     _lib = L
@@ -101,6 +106,28 @@ def _ptr(t):
     return None if t is None or t.numel() == 0 else t.data_ptr()
 
 
+class HitRecord:
+    """Device buffer in which a forward trace stores its per-chunk hit buffers so that the backward trace can
+    replay them instead of walking the BVH again (see `hit_record` in include/dst_api.h)."""
+
+    def __init__(self, H, W, mtd_alloc, blocks_per_wave, device):
+        header, waves = C.c_uint64(0), C.c_uint32(0)
+        lib = load_library()
+        lib.dst_hit_record_layout(H, W, mtd_alloc, 0, C.byref(header), C.byref(waves))
+        self.n_waves = max(1, waves.value)
+        self.blocks = max(1, int(self.n_waves * blocks_per_wave) + 1)
+        words = lib.dst_hit_record_layout(H, W, mtd_alloc, self.blocks, None, None)
+        self.words = torch.empty(words, dtype=torch.int64, device=device)
+        self.words[: header.value].zero_()
+
+    def requested_blocks(self):
+        """Blocks the forward trace asked for (waits for it to finish)."""
+        return int(self.words[0].item())
+
+    def complete(self):
+        return self.requested_blocks() <= self.blocks
+
+
 class OptiXStateWrapper:
     """Owner of the acceleration structure; keeps the reference's class name (ext.cpp:8) so callers need not
     change.  `pkg_dir` was where the reference looked for its PTX files and is ignored."""
@@ -114,6 +141,7 @@ class OptiXStateWrapper:
             raise RuntimeError("dst_create failed: no usable HIP device")
         self.device = torch.cuda.current_device()
         self.num_surfels = 0
+        self.record_blocks_per_wave = 6.0   # sizing estimate for hit records, raised when a record overflows
 
     def accel_info(self):
         info = DstAccelInfo()
@@ -179,11 +207,12 @@ def _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, col
 def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, background, means3D, shs, degree,
                   colors_precomp, others_precomp, opacities, scales, scale_modifier, rotations, transMat_precomp,
                   viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth, specular_threshold,
-                  counters=None, events=None):
+                  counters=None, events=None, hit_record=None):
     """Reference TraceSurfelsCUDA (trace_surfels.cpp:162-304): returns
     (out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights or None).
     Extras for measurement: `counters` (2 int64 on the device) receives the evaluated / composited hit totals;
-    `events` (two torch.cuda.Event) are recorded on the launch stream right around the kernel launch."""
+    `events` (two torch.cuda.Event) are recorded on the launch stream right around the kernel launch;
+    `hit_record` (a HitRecord) receives the hit buffers for a later replay by trace_surfels_backward."""
     p, keep = _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp,
                              others_precomp, opacities, scales, scale_modifier, rotations, max_trace_depth,
                              specular_threshold, start_from_first)
@@ -199,6 +228,8 @@ def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, backg
     p.mid_val = mid_val.data_ptr()
     p.a_weights = _ptr(a_weights)
     p.counters = _ptr(counters)
+    if hit_record is not None:
+        p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))
@@ -213,7 +244,7 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
                            transMat_precomp, viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth,
                            specular_threshold, out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val,
                            dL_dout_rgb, dL_dout_dpt, dL_dout_acc, dL_dout_norm, dL_dout_dist, dL_dout_aux,
-                           events=None):
+                           events=None, hit_record=None):
     """Reference TraceSurfelsBackwardCUDA (trace_surfels.cpp:307-464): returns (dL_dray_o, dL_dray_d, dL_dmeans3D,
     dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers, dL_dopacities, dL_dscales, dL_drotations,
     dL_dtransMat_precomp)."""
@@ -249,6 +280,12 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
     p.dL_dcolors, p.dL_dothers = dL_dcolors.data_ptr(), dL_dothers.data_ptr()
     p.dL_dopacities, p.dL_dscales, p.dL_drotations = (dL_dopacities.data_ptr(), dL_dscales.data_ptr(),
                                                       dL_drotations.data_ptr())
+    if hit_record is not None:
+        # replay only a complete record; an overflowed one means re-tracing (and a larger estimate next time)
+        asked = hit_record.requested_blocks()
+        ctx.record_blocks_per_wave = max(ctx.record_blocks_per_wave, 1.25 * asked / hit_record.n_waves)
+        if asked <= hit_record.blocks:
+            p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))

@@ -62,8 +62,14 @@ class _TraceSurfels(torch.autograd.Function):
         args = (optix_context, training, start_from_first, ray_o, ray_d, vertices, s.bg, means3D, shs, s.sh_degree,
                 colors_precomp, others_precomp, opacities, scales, s.scale_modifier, rotations,
                 cov3Ds_precomp) + _settings_args(s)
+        # when a backward pass will follow, the forward trace records its hit buffers for it
+        record = None
+        if any(ctx.needs_input_grad) and ray_o.dim() == 3 and ray_o.numel() > 0:
+            record = _C.HitRecord(ray_o.size(0), ray_o.size(1), max(_C.DEFAULT_MAX_TRACE_DEPTH, s.max_trace_depth),
+                                  optix_context.record_blocks_per_wave, ray_o.device)
         out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights = _guarded(
-            _C.trace_surfels, args, s.debug, "snapshot_fw.dump", "forward")
+            lambda *a: _C.trace_surfels(*a, hit_record=record), args, s.debug, "snapshot_fw.dump", "forward")
+        ctx.hit_record = record
 
         ctx.tracer_settings = s
         ctx.optix_context = optix_context
@@ -87,7 +93,8 @@ class _TraceSurfels(torch.autograd.Function):
                     out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val,
                     grad_out_rgb, grad_out_dpt, grad_out_acc, grad_out_norm, grad_out_dist, grad_out_aux)
         (g_ray_o, g_ray_d, g_means3D, g_grads3D, _g_grads3D_abs, g_shs, g_colors, g_others, g_opacities, g_scales,
-         g_rotations, g_cov3Ds) = _guarded(_C.trace_surfels_backward, args, s.debug, "snapshot_bw.dump", "backward")
+         g_rotations, g_cov3Ds) = _guarded(lambda *a: _C.trace_surfels_backward(*a, hit_record=ctx.hit_record), args,
+                                           s.debug, "snapshot_bw.dump", "backward")
 
         def like(grad, inp):  # an absent optional input (empty placeholder tensor) gets no gradient
             return grad if inp.numel() != 0 else None

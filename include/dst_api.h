@@ -77,6 +77,15 @@ typedef struct DstParams {
     float *a_weights;             /* (P,1), ACCUMULATED into: caller zero-fills; NULL when !training */
     /* optional forward statistics: counters[0] += entries evaluated, counters[1] += hits composited */
     unsigned long long *counters;
+    /* optional hit record (no counterpart in the reference): when non-NULL the forward trace stores every
+     * chunk's 16-entry hit buffer in it, and a backward trace given the same, complete record replays the
+     * buffers instead of walking the BVH again (same results, no traversal).  Device memory, 8-byte aligned,
+     * sized with dst_hit_record_layout(); the caller zero-fills the first header_words words before the
+     * forward call.  Word 0 then holds the number of blocks the forward trace asked for: if that exceeds
+     * hit_record_blocks the record is incomplete and must not be passed to the backward call. */
+    uint64_t *hit_record;
+    uint32_t hit_record_blocks;
+    uint32_t reserved0;
     /* upstream gradients (backward) */
     const float *dL_drgb, *dL_ddpt, *dL_dacc, *dL_ddist, *dL_dnorm, *dL_daux;
     /* gradient outputs; the per-surfel ones are ACCUMULATED into: caller zero-fills */
@@ -136,6 +145,12 @@ const char *dst_last_error(dst_ctx *ctx);
 int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info);
 int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_parent, uint32_t *leaf_parent,
                        uint32_t *sorted_keys, void *stream);
+
+/* Size in 8-byte words of a hit record with room for `blocks` chunk blocks, for an (H,W) ray grid traced with
+ * `mtd_alloc`.  Also returns the words of the header the caller must zero-fill, and the number of waves the
+ * grid is traced with (a forward trace at depth 0 asks for about 3-6 blocks per wave). */
+uint64_t dst_hit_record_layout(int32_t H, int32_t W, int32_t mtd_alloc, uint32_t blocks, uint64_t *header_words,
+                               uint32_t *n_waves);
 
 /* Library version string, and sizeof(DstParams) as compiled (lets a foreign-language binding
  * verify its own struct layout before the first launch). */

@@ -1,5 +1,6 @@
-"""Writes tests/golden/cube_p400.npz: inputs are regenerated from seeds, expected outputs come from the CPU
-oracle (brute-force hit enumeration, reference any-hit rule).  The reference ships no golden vectors and cannot be
+"""Writes tests/golden/cube_p400.npz: the inputs (generated from seeds here; stored, because vectorised exp / sin
+differ in the last bit between CPUs) and the expected outputs from the CPU oracle (brute-force hit
+enumeration, reference any-hit rule).  The reference ships no golden vectors and cannot be
 run here (it needs nvcc + OptiX), so this fixture pins the oracle against later drift, not against the reference.
 
     python tests/golden/make_golden.py
@@ -15,6 +16,16 @@ for p in (ROOT, os.path.join(ROOT, "diff-surfel-tracing_amd"), os.path.join(ROOT
     sys.path.insert(0, p)
 
 SPEC = dict(P=400, seed=11, H=24, W=24, view=1, aux=2, bg=(0.1, 0.2, 0.3), grad_seed=3)
+
+
+def load_inputs():
+    """The stored inputs of the fixture as torch tensors: (scene dict, ray_o, ray_d, upstream gradients)."""
+    import torch
+    z = np.load(os.path.join(HERE, "cube_p400.npz"))
+    sc = {k[3:]: torch.from_numpy(z[k]) for k in z.files if k.startswith("in_")}
+    o, d = sc.pop("ray_o"), sc.pop("ray_d")
+    ug = {k[3:]: torch.from_numpy(z[k]) for k in z.files if k.startswith("up_")}
+    return sc, o, d, ug
 
 
 def inputs():
@@ -34,7 +45,10 @@ def main():
     s = oracle_scene(O, sc, o, d, bg=SPEC["bg"])
     fwd = O.forward(s, O.HITS_BRUTE_LITERAL)
     bwd = O.backward(s, fwd, {k: v.numpy() for k, v in ug.items()}, O.HITS_BRUTE_LEXI)
-    out = {"fwd_" + k: v for k, v in fwd.items()}
+    out = {"in_" + k: v.numpy() for k, v in sc.items()}
+    out.update({"in_ray_o": o.numpy(), "in_ray_d": d.numpy()})
+    out.update({"up_" + k: v.numpy() for k, v in ug.items()})
+    out.update({"fwd_" + k: v for k, v in fwd.items()})
     out.update({"bwd_" + k: v for k, v in bwd.items()})
     np.savez_compressed(os.path.join(HERE, "cube_p400.npz"), **out)
     print("wrote", len(out), "arrays; composited hits per ray: mean %.1f max %d"

@@ -20,7 +20,7 @@ def golden():
 
 
 def test_oracle_reproduces_the_fixture(oracle, golden):
-    sc, o, d, ug = make_golden.inputs()
+    sc, o, d, ug = make_golden.load_inputs()
     s = oracle_scene(oracle, sc, o, d, bg=make_golden.SPEC["bg"])
     for mode in (oracle.HITS_BRUTE_LITERAL, oracle.HITS_BVH_LEXI):
         fwd = oracle.forward(s, mode)
@@ -35,7 +35,7 @@ def test_oracle_reproduces_the_fixture(oracle, golden):
 
 @pytest.mark.gpu
 def test_gpu_matches_the_fixture(tracer, golden):
-    sc, o, d, ug = make_golden.inputs()
+    sc, o, d, ug = make_golden.load_inputs()
     out, g = gpu_trace(tracer, sc, o, d, upstream=ug, bg=make_golden.SPEC["bg"])
     assert_forward_exact(out, {k[4:]: v for k, v in golden.items() if k.startswith("fwd_")})
     assert_close_sum(out["wet"], golden["fwd_wet"], 1e-5, "wet")

@@ -180,3 +180,56 @@ def test_config3_full_size_properties_and_sampled_parity(oracle, tracer):
         np.testing.assert_array_equal(got.view(np.uint32), ref[k].view(np.uint32), err_msg=k)
     assert ref["n_con"].mean() > 10
     del dev
+
+
+def test_backward_replays_the_forward_hit_record_or_retraces(oracle, tracer):
+    """The autograd path records the forward hit buffers and replays them in backward; a record that is too small
+    makes backward walk the BVH again.  Both must give the oracle's gradients, and an overflow raises the estimate."""
+    sc = S.scene_cube(P=6000, seed=4)
+    o, d = S.rays_cube(64, 64)
+    s = oracle_scene(oracle, sc, o, d)
+    ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
+    ug = upstream(64, 64, 2)
+    refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
+    ctx = tracer.optix_context
+    saved = ctx.record_blocks_per_wave
+    try:
+        for estimate in (8.0, 0.01):
+            ctx.record_blocks_per_wave = estimate
+            out, g = gpu_trace(tracer, sc, o, d, upstream=ug)
+            assert_forward_exact(out, ref)
+            for k in ("ray_o", "ray_d", "means3D", "grads3D", "shs", "opacities", "scales", "rotations"):
+                assert_close_sum(g[k], refg[k], GRAD_REL, k)
+        assert ctx.record_blocks_per_wave > 1.0   # learnt from the overflow
+    finally:
+        ctx.record_blocks_per_wave = max(saved, ctx.record_blocks_per_wave)
+
+
+def test_raw_launcher_calls_without_a_record(oracle, tracer):
+    """The four `_C` callables with exactly the reference's positional arguments (24 and 36)."""
+    import diff_surfel_tracing._C as binding
+    sc = S.scene_cube(P=3000, seed=6)
+    o, d = S.rays_cube(32, 40)
+    dev = "cuda"
+    g = {k: v.to(dev) for k, v in sc.items()}
+    ctx = tracer.optix_context
+    binding.build_acceleration_structure(ctx, g["vertices"], g["faces"], True)
+    e, eye, z3 = torch.empty(0, device=dev), torch.eye(4, device=dev), torch.zeros(3, device=dev)
+    common = (g["vertices"], z3, g["means3D"], g["shs"], 3, e, e, g["opacities"], g["scales"], 1.0, g["rotations"], e,
+              eye, eye, z3, False, False, 0, 0.0)
+    fwd = binding.trace_surfels(ctx, True, True, o.to(dev), d.to(dev), *common)
+    assert len(fwd) == 8
+    ug = upstream(32, 40, 2)
+    ups = [ug[k].to(dev) for k in ("rgb", "dpt", "acc", "norm")] + [torch.zeros(32, 40, 1, device=dev), ug["aux"].to(dev)]
+    bwd = binding.trace_surfels_backward(ctx, True, o.to(dev), d.to(dev), *common, *fwd[:7], *ups)
+    assert len(bwd) == 12
+    s = oracle_scene(oracle, sc, o, d)
+    ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
+    refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
+    np.testing.assert_array_equal(fwd[0].cpu().numpy(), ref["rgb"])
+    names = ("ray_o", "ray_d", "means3D", "grads3D", None, "shs", "colors_precomp", None, "opacities", "scales",
+             "rotations", None)
+    for t, k in zip(bwd, names):
+        if k is not None:
+            assert_close_sum(t.cpu().numpy(), refg[k], GRAD_REL, k)
+    assert bwd[4].abs().max() == 0 and bwd[11].shape == (3000, 9) and bwd[11].abs().max() == 0
