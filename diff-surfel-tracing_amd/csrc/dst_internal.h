@@ -36,12 +36,16 @@ struct alignas(128) DstWideNode {
     uint32_t pad[3];
 };
 
-// Leaf = one surfel quad in Morton order: corners A,B,C,D (triangles ABC and BCD) and the surfel id.
-struct alignas(64) DstLeaf {
+// Leaf = one surfel quad in Morton order: corners A,B,C,D (triangles ABC and BCD), the two plane normals
+// n0 = (B-A)x(C-A), n1 = (C-B)x(D-B) as the hit test defines them, and the surfel id.  80 bytes, fetched
+// once per wave.
+struct alignas(16) DstLeaf {
     float A[3], B[3], C[3], D[3];
+    float n0[3], n1[3];
     uint32_t g;
-    uint32_t pad[3];
+    uint32_t pad;
 };
+static_assert(sizeof(DstLeaf) == 80, "leaf records are 20 dwords");
 
 struct DstBounds {          // device-resident reduction targets, order-preserving uint encoding
     uint32_t lo[3], hi[3];  // centroid bounds

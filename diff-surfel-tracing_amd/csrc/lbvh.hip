@@ -275,7 +275,8 @@ __global__ void k_karras(const uint32_t *__restrict__ keys, DstNode *__restrict_
     if (i == 0) node_parent[0] = DST_NO_PARENT;
 }
 
-// Leaf records in Morton order (also the whole of a refit's geometry update).
+// Leaf records in Morton order (also the whole of a refit's geometry update).  The plane normals use the
+// fused form the hit test is defined with: cross(x,y).x = fma(x.y, y.z, -(x.z*y.y)), and so on.
 __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
                             const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves, uint32_t n) {
     uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -283,19 +284,43 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
     uint32_t g = sorted_ids[i];
     int4 q = quad_ids[g];
     const int ids[4] = {q.x, q.y, q.z, q.w};
-    float out[16];
+    float c[4][3];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const float *v = vertices + (size_t)ids[k] * 3;
-        out[3 * k + 0] = v[0];
-        out[3 * k + 1] = v[1];
-        out[3 * k + 2] = v[2];
+        c[k][0] = v[0];
+        c[k][1] = v[1];
+        c[k][2] = v[2];
     }
-    out[12] = __uint_as_float(g);
-    out[13] = out[14] = out[15] = 0.f;
+    auto cross_f = [](const float *x, const float *y, float *out) {
+        out[0] = __builtin_fmaf(x[1], y[2], -(x[2] * y[1]));
+        out[1] = __builtin_fmaf(x[2], y[0], -(x[0] * y[2]));
+        out[2] = __builtin_fmaf(x[0], y[1], -(x[1] * y[0]));
+    };
+    float e1[3], e2[3], f1[3], f2[3], n0[3], n1[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        e1[a] = c[1][a] - c[0][a];   // B - A
+        e2[a] = c[2][a] - c[0][a];   // C - A
+        f1[a] = c[2][a] - c[1][a];   // C - B
+        f2[a] = c[3][a] - c[1][a];   // D - B
+    }
+    cross_f(e1, e2, n0);
+    cross_f(f1, f2, n1);
+    float out[20];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        for (int a = 0; a < 3; ++a) out[3 * k + a] = c[k][a];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        out[12 + a] = n0[a];
+        out[15 + a] = n1[a];
+    }
+    out[18] = __uint_as_float(g);
+    out[19] = 0.f;
     float4 *dst = reinterpret_cast<float4 *>(&leaves[i]);
 #pragma unroll
-    for (int k = 0; k < 4; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
+    for (int k = 0; k < 5; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
 }
 
 // Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes.

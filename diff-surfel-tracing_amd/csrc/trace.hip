@@ -101,15 +101,22 @@ __device__ __forceinline__ F3 sh_color(int deg, const float *__restrict__ sh, F3
 }
 
 // ---- ray / quad -----------------------------------------------------------------------------------------
-__device__ __forceinline__ float triple(F3 d, F3 x, F3 y) {
-    return d.x * (x.y * y.z - x.z * y.y) + d.y * (x.z * y.x - x.x * y.z) + d.z * (x.x * y.y - x.y * y.x);
+// Products feeding a difference or a running sum are fused here BY DEFINITION (explicit fma, one rounding);
+// the CPU statement of the same test uses the same calls, so both sides produce the same bits.
+__device__ __forceinline__ F3 cross_f(F3 x, F3 y) {
+    return F3{__builtin_fmaf(x.y, y.z, -(x.z * y.y)), __builtin_fmaf(x.z, y.x, -(x.x * y.z)),
+              __builtin_fmaf(x.x, y.y, -(x.y * y.x))};
 }
+__device__ __forceinline__ float dot_f(F3 a, F3 b) {
+    return __builtin_fmaf(a.z, b.z, __builtin_fmaf(a.y, b.y, a.x * b.x));
+}
+__device__ __forceinline__ float triple(F3 d, F3 x, F3 y) { return dot_f(d, cross_f(x, y)); }
 __device__ __forceinline__ bool same_sign(float a, float b, float c) {
     return (a >= 0.f && b >= 0.f && c >= 0.f) || (a <= 0.f && b <= 0.f && c <= 0.f);
 }
-// Quad = triangles ABC and BCD.  Signed-volume edge tests in origin-relative coordinates, then
-// t = n.(v1-o) / n.d on the plane of the triangle that was hit.
-__device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 B, F3 C, F3 Dv, float &t, uint32_t &tri) {
+// Quad = triangles ABC and BCD with plane normals n0, n1.  Signed-volume edge tests in origin-relative
+// coordinates, then t = n.(v1-o) / n.d on the plane of the triangle that was hit.
+__device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 B, F3 C, F3 Dv, F3 n0, F3 n1, float &t, uint32_t &tri) {
     F3 a = A - o, b = B - o, c = C - o, e = Dv - o;
     float u0 = triple(d, b, c);
     float u1 = triple(d, c, a);
@@ -119,13 +126,11 @@ __device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 B, F3 C, F3 Dv, fl
     float w1 = triple(d, e, b);
     bool in1 = same_sign(w0, w1, u0);
     if (!(in0 || in1)) return false;
-    F3 n0 = cross(B - A, C - A);
-    F3 n1 = cross(C - B, Dv - B);
     F3 n = in0 ? n0 : n1;
     F3 k = in0 ? a : b;
     tri = in0 ? 0u : 1u;
-    float p = dot(n, k);
-    float q = dot(n, d);
+    float p = dot_f(n, k);
+    float q = dot_f(n, d);
     t = p / q;
     return (t > 0.0f) && (t < kInfDepth);
 }
@@ -226,17 +231,15 @@ __device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool 
                                           , WaveStats &ws
 #endif
 ) {
-    uint32_t L[13];
-    load_uniform<13>(leaf, L);
+    uint32_t L[19];
+    load_uniform<19>(leaf, L);
     STAT(ws.leaves++;)
-    F3 A = f3(__uint_as_float(L[0]), __uint_as_float(L[1]), __uint_as_float(L[2]));
-    F3 B = f3(__uint_as_float(L[3]), __uint_as_float(L[4]), __uint_as_float(L[5]));
-    F3 C = f3(__uint_as_float(L[6]), __uint_as_float(L[7]), __uint_as_float(L[8]));
-    F3 Dv = f3(__uint_as_float(L[9]), __uint_as_float(L[10]), __uint_as_float(L[11]));
+#define LF3(k) f3(__uint_as_float(L[k]), __uint_as_float(L[(k) + 1]), __uint_as_float(L[(k) + 2]))
     float t = 0.f;
     uint32_t tri = 0u;
-    const bool hit = active && ray_quad(o, d, A, B, C, Dv, t, tri);
-    const uint64_t x = kb_pack(t, 2u * L[12] + tri);
+    const bool hit = active && ray_quad(o, d, LF3(0), LF3(3), LF3(6), LF3(9), LF3(12), LF3(15), t, tri);
+#undef LF3
+    const uint64_t x = kb_pack(t, 2u * L[18] + tri);
     const bool adm = hit && (x < buf.e[kChunk - 1]);
     if (__ballot(adm) != 0ull) {
         STAT(ws.leaf_any++;)

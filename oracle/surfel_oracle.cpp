@@ -25,8 +25,9 @@
  * itself is UNPINNED:
  *   - the set of hits of a ray: every surfel quad (two triangles sharing the
  *     edge B-C) is tested with signed-volume edge functions in ray-origin
- *     relative coordinates; at most one hit per quad; triangle 0 wins ties on
- *     the shared edge;
+ *     relative coordinates (cross and dot products with fused multiply-adds,
+ *     written out in ray_quad()); at most one hit per quad; triangle 0 wins
+ *     ties on the shared edge;
  *   - the hit parameter: t = n.(v1-o) / n.d with n = (v2-v1)x(v3-v1) of the hit
  *     triangle (the formula backward.cu:256-262 differentiates), accepted for
  *     0 < t < 1e16;
@@ -37,8 +38,9 @@
  * exactly-rounded IEEE sequences so that results are reproducible bit for bit
  * on any IEEE machine: rsqrtf(x) := 1/sqrtf(x), exp(x) := oracle_expf(x)
  * (Cody-Waite + degree-6 polynomial, <= 1 ulp from the true value on the range
- * used).  All arithmetic is fp32, evaluated left to right as written, never
- * contracted into fused multiply-adds (compile with -ffp-contract=off).
+ * used).  All arithmetic is fp32, evaluated left to right as written and never
+ * contracted by the compiler (compile with -ffp-contract=off); the only fused
+ * multiply-adds are the explicit std::fmaf calls of the ray/quad test.
  *
  * Deviations from the literal reference, all switchable or unreachable there:
  *   - a buffer entry skipped because its surfel equals the last contributing
@@ -234,9 +236,13 @@ inline void splat_uv(const float *mean, const float *scale, const float *rot, V3
 }
 
 // ---- ray / surfel-quad test (defined here, see the header comment) ---------------------------
-inline float triple(V3 d, V3 x, V3 y) {
-    return d.x * (x.y * y.z - x.z * y.y) + d.y * (x.z * y.x - x.x * y.z) + d.z * (x.x * y.y - x.y * y.x);
+// Products that feed a difference or a running sum are fused (std::fmaf, one rounding), exactly as written:
+// the fused form is part of the definition, so any IEEE machine reproduces it bit for bit.
+inline V3 cross_f(V3 x, V3 y) {
+    return V3{std::fmaf(x.y, y.z, -(x.z * y.y)), std::fmaf(x.z, y.x, -(x.x * y.z)), std::fmaf(x.x, y.y, -(x.y * y.x))};
 }
+inline float dot_f(V3 a, V3 b) { return std::fmaf(a.z, b.z, std::fmaf(a.y, b.y, a.x * b.x)); }
+inline float triple(V3 d, V3 x, V3 y) { return dot_f(d, cross_f(x, y)); }
 inline bool same_sign(float a, float b, float c) {
     return (a >= 0.f && b >= 0.f && c >= 0.f) || (a <= 0.f && b <= 0.f && c <= 0.f);
 }
@@ -247,19 +253,19 @@ inline bool ray_quad(V3 o, V3 d, V3 A, V3 B, V3 C, V3 Dv, float &t, int &tri) {
     float u2 = triple(d, a, b);
     V3 n, k;
     if (same_sign(u0, u1, u2)) {
-        n = cross(B - A, C - A);
+        n = cross_f(B - A, C - A);
         k = a;
         tri = 0;
     } else {
         float w0 = triple(d, c, e);
         float w1 = triple(d, e, b);
         if (!same_sign(w0, w1, u0)) return false;
-        n = cross(C - B, Dv - B);
+        n = cross_f(C - B, Dv - B);
         k = b;
         tri = 1;
     }
-    float p = dot(n, k);
-    float q = dot(n, d);
+    float p = dot_f(n, k);
+    float q = dot_f(n, d);
     t = p / q;
     return (t > 0.0f) && (t < kInfDepth);
 }

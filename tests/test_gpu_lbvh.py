@@ -13,14 +13,15 @@ LEAF = 0x80000000
 
 NODE = np.dtype([("lo0", "<f4", 3), ("hi0", "<f4", 3), ("lo1", "<f4", 3), ("hi1", "<f4", 3), ("c0", "<u4"),
                  ("c1", "<u4"), ("first", "<u4"), ("last", "<u4")])
-LEAFT = np.dtype([("A", "<f4", 3), ("B", "<f4", 3), ("C", "<f4", 3), ("D", "<f4", 3), ("g", "<u4"), ("pad", "<u4", 3)])
+LEAFT = np.dtype([("A", "<f4", 3), ("B", "<f4", 3), ("C", "<f4", 3), ("D", "<f4", 3), ("n0", "<f4", 3),
+                  ("n1", "<f4", 3), ("g", "<u4"), ("pad", "<u4")])
 
 
 def download(tracer):
     import diff_surfel_tracing._C as binding
     ctx = tracer.optix_context
     info = ctx.accel_info()
-    assert info.node_bytes == NODE.itemsize == 64 and info.leaf_bytes == LEAFT.itemsize == 64
+    assert info.node_bytes == NODE.itemsize == 64 and info.leaf_bytes == LEAFT.itemsize == 80
     n = info.n_surfels
     nodes = np.zeros(max(n - 1, 1), NODE)
     leaves = np.zeros(n, LEAFT)
@@ -39,6 +40,9 @@ def check_tree(info, nodes, leaves, npar, lpar, keys, vertices):
     V = vertices.reshape(n, 4, 3)
     for name, k in (("A", 0), ("B", 1), ("C", 2), ("D", 3)):
         np.testing.assert_array_equal(leaves[name], V[leaves["g"], k])
+    A, B, C, D = (leaves[c].astype(np.float64) for c in "ABCD")
+    np.testing.assert_allclose(leaves["n0"], np.cross(B - A, C - A), rtol=1e-4, atol=1e-7)   # plane normals
+    np.testing.assert_allclose(leaves["n1"], np.cross(C - B, D - B), rtol=1e-4, atol=1e-7)
     llo = np.minimum.reduce([leaves[c] for c in "ABCD"])
     lhi = np.maximum.reduce([leaves[c] for c in "ABCD"])
     # walk from the root: every node and leaf reached once, parents consistent, boxes = exact union of content
