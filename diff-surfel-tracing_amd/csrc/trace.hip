@@ -76,6 +76,8 @@ __device__ __forceinline__ void quat_rows(const float q0, const float q1, const 
 // SH colour of one surfel in direction d (reference forward.cu:18-58); clamp flags for backward.
 __device__ __forceinline__ F3 sh_color(int deg, const float *__restrict__ sh, F3 d, bool (&neg)[3]) {
 #define SHC(j) f3(sh[3 * (j)], sh[3 * (j) + 1], sh[3 * (j) + 2])
+
+
     F3 r = SH0 * SHC(0);
     if (deg > 0) {
         float x = d.x, y = d.y, z = d.z;
@@ -334,7 +336,11 @@ __device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v);
 // are first summed in an LDS hash table (one row of columns per surfel, LDS atomics) and written to
 // global memory once per surfel and block when the block ends.  A surfel that finds no free row within a
 // few probes goes straight to global atomics, so the table can never be wrong, only less effective.
-constexpr int kTableRows = 256;                 // power of two
+#ifndef DST_TABLE_ROWS_LOG2
+#define DST_TABLE_ROWS_LOG2 7
+#endif
+constexpr int kTableRowsLog2 = DST_TABLE_ROWS_LOG2;
+constexpr int kTableRows = 1 << kTableRowsLog2;
 constexpr uint32_t kEmptyKey = 0xFFFFFFFFu;
 constexpr int kMaxProbe = 8;
 // row columns: colour 0-2, opacity 3, scales 4-5, rotation 6-9, mean 10-12, densification mean 13-15,
@@ -438,8 +444,7 @@ struct GradSink {
 // Find or claim the table row of surfel g.
 template <int AUXM>
 __device__ __forceinline__ float *table_row(uint32_t *keys, float *rows, uint32_t g) {
-    uint32_t slot = (g * 2654435761u) >> (32 - 8);
-    static_assert(kTableRows == 256, "hash shift assumes 256 rows");
+    uint32_t slot = (g * 2654435761u) >> (32 - kTableRowsLog2);
 #pragma unroll 1
     for (int probe = 0; probe < kMaxProbe; ++probe) {
         uint32_t k = __hip_atomic_load(keys + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -655,17 +660,16 @@ __device__ __forceinline__ void rec_store(const RecView &rv, int bounce, uint32_
     prev = blk;
 }
 
-// Backward: fetch the next chunk of this wave's bounce.  Returns false when the chain ends early.
-__device__ __forceinline__ bool rec_load(const RecView &rv, uint32_t &cur, KBuf &buf, uint32_t &cnt) {
-    if (cur == 0u || cur > rv.capacity) return false;
+// Backward: locate the next chunk of this wave's bounce; its entries are then read one slot at a time.
+// Returns nullptr when the chain ends early.
+__device__ __forceinline__ const uint64_t *rec_open(const RecView &rv, uint32_t &cur, uint32_t &cnt) {
+    if (cur == 0u || cur > rv.capacity) return nullptr;
     const uint32_t lane = __lane_id();
     const uint64_t *b = rv.blocks + (size_t)(cur - 1u) * kRecBlockWords;
-#pragma unroll
-    for (int k = 0; k < kChunk; ++k) buf.e[k] = b[k * DST_WAVE + lane];
     const uint32_t *cnts = reinterpret_cast<const uint32_t *>(b + kChunk * DST_WAVE);
     cnt = cnts[lane];
     cur = __builtin_amdgcn_readfirstlane(cnts[DST_WAVE]);
-    return true;
+    return b;
 }
 
 // One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
@@ -694,8 +698,13 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     while (__ballot(live) != 0ull) {
         uint32_t cnt = 0;
         STAT(ws.chunks++; unsigned long long c0 = __builtin_readcyclecounter();)
+        // Where the compositing loop below takes its entries from: the recorded block, one slot at a time
+        // (backward replay: no buffer registers at all), or the register buffer the traversal just filled.
+        const uint64_t *rec_block = nullptr;
+        const uint32_t lane_ = __lane_id();
         if (REC && BWD) {
-            if (!rec_load(rv, rec_pos, buf, cnt)) break;   // cannot happen with a complete record
+            rec_block = rec_open(rv, rec_pos, cnt);
+            if (rec_block == nullptr) break;   // cannot happen with a complete record
         } else {
             kbuf_reset(buf);
             packet_knn(acc, max_abs, ot, rd, live, buf, cnt WSP);
@@ -704,15 +713,21 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
         int here = 0;
         bool stop = false;
+#pragma unroll 1
         for (int it = 0; it < kChunk; ++it) {
             const bool on = live && !stop && (uint32_t)it < cnt;
             if (__ballot(on) == 0ull) break;
-            // pop the front entry; the rest moves up (consumed slots need no reset: the buffer is
-            // rebuilt from scratch for the next chunk)
-            const float e_t = kb_t(buf.e[0]);
-            const uint32_t e_i = kb_idx(buf.e[0]);
+            // next entry in depth order (consumed slots need no reset: the buffer is rebuilt for every chunk)
+            uint64_t e;
+            if (REC && BWD) {
+                e = rec_block[it * DST_WAVE + lane_];
+            } else {
+                e = buf.e[0];
 #pragma unroll
-            for (int k = 0; k < kChunk - 1; ++k) buf.e[k] = buf.e[k + 1];
+                for (int k = 0; k < kChunk - 1; ++k) buf.e[k] = buf.e[k + 1];
+            }
+            const float e_t = kb_t(e);
+            const uint32_t e_i = kb_idx(e);
             // ---- phase 1 (per lane): evaluate the entry, decide, composite ------------------------------
             bool did = false;          // this lane composited a hit in this iteration
             int g = 0;
@@ -842,9 +857,8 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
 }
 
 template <bool BWD, int AUXM, bool REC>
-__global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstParams p, const DstAccelView acc,
-                                                                     int tw_log2, int th_log2, uint32_t tiles_x,
-                                                                     uint32_t tiles_y, uint32_t btiles_x) {
+__device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
+                                           uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     __shared__ uint32_t s_keys[BWD ? kTableRows : 1];
@@ -858,16 +872,21 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
         __syncthreads();
     }
     const uint32_t wv = threadIdx.x / DST_WAVE;
+    // Blocks keep the dispatch order (row-major over the 16x16 pixel tiles).  Re-numbering them so that each of
+    // the 8 XCDs owns a band or whole rows of the image was measured and is slower on the 1080p room scene
+    // (+15 % / +8 % forward): the chip then works on 8 distant image regions at once and the shared last-level
+    // cache sees 8 times more distinct BVH data, which costs more than the per-XCD L2 gains.
+    const uint32_t bid = blockIdx.x;
     RecView rv = {nullptr, nullptr, nullptr, 0u};
     if (REC) {
         const uint32_t n_waves = gridDim.x * kWavesPerBlock, slots_ = (uint32_t)p.mtd_alloc + 1u;
         const uint64_t dir_words = ((uint64_t)n_waves * slots_ + 1u) / 2u;
         rv.base = p.hit_record;
-        rv.dir = reinterpret_cast<uint32_t *>(p.hit_record + 2) + (size_t)(blockIdx.x * kWavesPerBlock + wv) * slots_;
+        rv.dir = reinterpret_cast<uint32_t *>(p.hit_record + 2) + (size_t)(bid * kWavesPerBlock + wv) * slots_;
         rv.blocks = p.hit_record + 2 + dir_words;
         rv.capacity = p.hit_record_blocks;
     }
-    const uint32_t ty = 2u * (blockIdx.x / btiles_x) + (wv >> 1), tx = 2u * (blockIdx.x % btiles_x) + (wv & 1u);
+    const uint32_t ty = 2u * (bid / btiles_x) + (wv >> 1), tx = 2u * (bid % btiles_x) + (wv & 1u);
     const bool wave_on = ty < tiles_y && tx < tiles_x;
     if (!BWD && !wave_on) return;   // the backward kernel keeps every wave for the block-wide flush below
     const uint32_t lane = threadIdx.x % DST_WAVE;
@@ -1061,6 +1080,27 @@ __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) void k_trace(const DstPar
     }
 }
 
+// The two entry kernels differ only in the occupancy the register allocator is told to aim for: both are
+// bound by the latency of dependent fetches, so waves in flight matter more than a few spilled values.
+#ifndef DST_FWD_WAVES
+#define DST_FWD_WAVES 4
+#endif
+#ifndef DST_BWD_WAVES
+#define DST_BWD_WAVES 3
+#endif
+template <int AUXM, bool REC>
+__global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
+void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
+                 uint32_t tiles_y, uint32_t btiles_x) {
+    trace_body<false, AUXM, REC>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+}
+template <int AUXM, bool REC>
+__global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
+void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
+                 uint32_t tiles_y, uint32_t btiles_x) {
+    trace_body<true, AUXM, REC>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+}
+
 struct TileGrid {
     int tw_log2, th_log2;
     uint32_t tiles_x, tiles_y, btiles_x, btiles_y;
@@ -1082,15 +1122,19 @@ TileGrid tile_grid(int H, int W) {
 template <bool BWD, bool REC>
 void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipStream_t stream) {
     dim3 grid(t.btiles_x * t.btiles_y), block(kWavesPerBlock * DST_WAVE);
-    if (p.aux <= 2)
-        hipLaunchKernelGGL((k_trace<BWD, 2, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2, t.tiles_x,
-                           t.tiles_y, t.btiles_x);
-    else if (p.aux <= 4)
-        hipLaunchKernelGGL((k_trace<BWD, 4, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2, t.tiles_x,
-                           t.tiles_y, t.btiles_x);
-    else
-        hipLaunchKernelGGL((k_trace<BWD, 8, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2, t.tiles_x,
-                           t.tiles_y, t.btiles_x);
+#define DST_LAUNCH(AUX)                                                                                            \
+    do {                                                                                                           \
+        if (BWD)                                                                                                   \
+            hipLaunchKernelGGL((k_trace_bwd<AUX, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2,      \
+                               t.tiles_x, t.tiles_y, t.btiles_x);                                                  \
+        else                                                                                                       \
+            hipLaunchKernelGGL((k_trace_fwd<AUX, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2,      \
+                               t.tiles_x, t.tiles_y, t.btiles_x);                                                  \
+    } while (0)
+    if (p.aux <= 2) DST_LAUNCH(2);
+    else if (p.aux <= 4) DST_LAUNCH(4);
+    else DST_LAUNCH(8);
+#undef DST_LAUNCH
 }
 
 }  // namespace
