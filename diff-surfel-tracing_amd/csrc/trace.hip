@@ -176,18 +176,22 @@ __device__ __forceinline__ RaySlab make_slab(F3 o, F3 d, float max_abs) {
     return s;
 }
 
-// Entry distance of the ray into the widened box; the box is hit iff the result <= tmax (and tmax >= 0).
-__device__ __forceinline__ bool slab_hit(const RaySlab &s, const uint32_t *box /* lo[3],hi[3] */, float tmax, float &tn) {
-    float lx = __uint_as_float(box[0]), ly = __uint_as_float(box[1]), lz = __uint_as_float(box[2]);
-    float hx = __uint_as_float(box[3]), hy = __uint_as_float(box[4]), hz = __uint_as_float(box[5]);
-    float ax = __builtin_fmaf(lx, s.ix, s.nx), bx = __builtin_fmaf(hx, s.ix, s.nx);
-    float ay = __builtin_fmaf(ly, s.iy, s.ny), by = __builtin_fmaf(hy, s.iy, s.ny);
-    float az = __builtin_fmaf(lz, s.iz, s.nz), bz = __builtin_fmaf(hz, s.iz, s.nz);
-    float n0 = __builtin_fminf(ax, bx) - s.wx, f0 = __builtin_fmaxf(ax, bx) + s.wx;
-    float n1 = __builtin_fminf(ay, by) - s.wy, f1 = __builtin_fmaxf(ay, by) + s.wy;
-    float n2 = __builtin_fminf(az, bz) - s.wz, f2 = __builtin_fmaxf(az, bz) + s.wz;
-    tn = __builtin_fmaxf(__builtin_fmaxf(n0, n1), __builtin_fmaxf(n2, 0.0f));
-    float tf = __builtin_fminf(__builtin_fminf(f0, f1), __builtin_fminf(f2, tmax));
+// Conservative slab test for a packet whose lanes all have the same direction signs: the near and far plane of
+// each axis are then the same box faces for all lanes, picked once per wave, and the widening folds into the
+// offsets.  The box is hit iff the entry distance tn <= min(exit distance, tmax); tmax < 0 disables a lane.
+struct RaySlabFast {
+    float ix, iy, iz;
+    float cnx, cny, cnz;   // -o/d - widening: added to (near face)/d
+    float cfx, cfy, cfz;   // -o/d + widening: added to (far face)/d
+};
+__device__ __forceinline__ bool slab_hit_fast(const RaySlabFast &s, float nx, float ny, float nz, float fx, float fy,
+                                              float fz, float tmax, float &tn) {
+    const float a = __builtin_fmaf(nx, s.ix, s.cnx), b = __builtin_fmaf(ny, s.iy, s.cny),
+                c = __builtin_fmaf(nz, s.iz, s.cnz);
+    const float e = __builtin_fmaf(fx, s.ix, s.cfx), f = __builtin_fmaf(fy, s.iy, s.cfy),
+                g = __builtin_fmaf(fz, s.iz, s.cfz);
+    tn = __builtin_fmaxf(__builtin_fmaxf(a, b), __builtin_fmaxf(c, 0.0f));
+    const float tf = __builtin_fminf(__builtin_fminf(e, f), __builtin_fminf(g, tmax));
     return tn <= tf;
 }
 
@@ -254,20 +258,26 @@ __device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool 
 // to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow: nodes and quads
 // are fetched once per wave, the stack is three VGPRs addressed by lane (192 entries: the binary hierarchy
 // is at most 62 levels deep and each 4-wide step defers at most three children).
-__device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
-                                           uint32_t &cnt
+// All active lanes share the direction signs `sgn` (bit a set = axis a negative), see slab_hit_fast.
+__device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySlab &slab, uint32_t sgn, F3 o, F3 d,
+                                            bool active, int rep, KBuf &buf, uint32_t &cnt
 #ifdef DST_STATS
-                                           , WaveStats &ws
+                                            , WaveStats &ws
 #define WSP , ws
 #else
 #define WSP
 #endif
 ) {
-    const uint64_t live = __ballot(active);
-    if (live == 0ull) return;
-    const RaySlab slab = make_slab(o, d, max_abs);
     const uint32_t lane = __lane_id();
-    const int rep = __builtin_ctzll(live);   // the lane whose entry distances order the children
+    RaySlabFast fs;
+    // byte offsets of the near / far face arrays inside a wide node (lox 0, loy 16, loz 32, hix 48, hiy 64, hiz 80)
+    uint32_t onx = 0, ony = 16, onz = 32, ofx = 48, ofy = 64, ofz = 80;
+    fs.ix = slab.ix; fs.iy = slab.iy; fs.iz = slab.iz;
+    fs.cnx = slab.nx - slab.wx; fs.cny = slab.ny - slab.wy; fs.cnz = slab.nz - slab.wz;
+    fs.cfx = slab.nx + slab.wx; fs.cfy = slab.ny + slab.wy; fs.cfz = slab.nz + slab.wz;
+    if (sgn & 1u) { onx = 48; ofx = 0; }
+    if (sgn & 2u) { ony = 64; ofy = 16; }
+    if (sgn & 4u) { onz = 80; ofz = 32; }
     uint32_t stack0 = 0u, stack1 = 0u, stack2 = 0u;
     int sp = 0;
     uint32_t ref = acc.root;
@@ -280,24 +290,31 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
                 test_leaf(&acc.leaves[first + q], o, d, active, buf, cnt WSP);
         } else {
             if (ref + 1u >= acc.n_leaves) break;   // not a node of this hierarchy
-            uint32_t Nd[29];
-            load_uniform<29>(&acc.wide[ref], Nd);
+            const char *node = reinterpret_cast<const char *>(&acc.wide[ref]);
             STAT(ws.nodes++;)
             const float tmax = active ? kb_t(buf.e[kChunk - 1]) : -1.0f;
-            const uint32_t n_child = Nd[28];
-            uint32_t key[DST_WIDE], cref[DST_WIDE];
+            uint32_t key[DST_WIDE], cref[DST_WIDE], tail[5];
+            load_uniform<5>(node + 96, tail);      // ref[4], count
+            const uint32_t n_child = tail[4];
             int n_push = 0;
+            {
+                uint32_t NX[4], NY[4], NZ[4], FX[4], FY[4], FZ[4];
+                load_uniform<4>(node + onx, NX); load_uniform<4>(node + ony, NY); load_uniform<4>(node + onz, NZ);
+                load_uniform<4>(node + ofx, FX); load_uniform<4>(node + ofy, FY); load_uniform<4>(node + ofz, FZ);
 #pragma unroll
-            for (int k = 0; k < DST_WIDE; ++k) {
-                const uint32_t box[6] = {Nd[k], Nd[4 + k], Nd[8 + k], Nd[12 + k], Nd[16 + k], Nd[20 + k]};
-                float tn;
-                const bool h = slab_hit(slab, box, tmax, tn) && (uint32_t)k < n_child;   // unused slots are never entered
-                const bool any = __ballot(h) != 0ull;
-                // entry distance of the representative lane (non-negative, so its bits order like the value)
-                const uint32_t kk = __builtin_amdgcn_readlane(h ? __float_as_uint(tn) : 0x7F800000u, rep);
-                key[k] = any ? kk : 0xFFFFFFFFu;
-                cref[k] = Nd[24 + k];
-                n_push += any ? 1 : 0;
+                for (int k = 0; k < DST_WIDE; ++k) {
+                    float tn;
+                    const bool h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
+                                                 __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
+                                                 __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn) &&
+                                   (uint32_t)k < n_child;   // unused slots are never entered
+                    const bool any = __ballot(h) != 0ull;
+                    // entry distance of the representative lane (non-negative, so its bits order like the value)
+                    const uint32_t kk = __builtin_amdgcn_readlane(h ? __float_as_uint(tn) : 0x7F800000u, rep);
+                    key[k] = any ? kk : 0xFFFFFFFFu;
+                    cref[k] = tail[k];
+                    n_push += any ? 1 : 0;
+                }
             }
             if (n_push > 0) {
                 // sort the four (key, ref) pairs, nearest first; children nobody wants carry the largest key
@@ -326,6 +343,29 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
         if (sp == 0) break;
         --sp;
         ref = __builtin_amdgcn_readlane(sp < 64 ? stack0 : (sp < 128 ? stack1 : stack2), sp & 63);
+    }
+}
+
+__device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
+                                           uint32_t &cnt
+#ifdef DST_STATS
+                                           , WaveStats &ws
+#endif
+) {
+    const uint64_t live = __ballot(active);
+    if (live == 0ull) return;
+    const RaySlab slab = make_slab(o, d, max_abs);
+    // The walk assumes one set of direction signs per packet (the near face of every box is then the same for
+    // all lanes).  A wave whose rays straddle an axis plane (about 1 % of the tiles of a pinhole image) is
+    // walked once per sign class present, each time with the lanes of that class only.
+    const uint32_t my_sgn = (slab.ix < 0.f ? 1u : 0u) | (slab.iy < 0.f ? 2u : 0u) | (slab.iz < 0.f ? 4u : 0u);
+    uint64_t todo = live;
+    while (todo != 0ull) {
+        const int rep = __builtin_ctzll(todo);   // also the lane whose entry distances order the children
+        const uint32_t sgn = __builtin_amdgcn_readlane(my_sgn, rep);
+        const bool mine = active && my_sgn == sgn;
+        todo &= ~__ballot(mine);
+        packet_walk(acc, slab, sgn, o, d, mine, rep, buf, cnt WSP);
     }
 }
 
