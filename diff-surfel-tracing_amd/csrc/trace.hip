@@ -423,6 +423,28 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));   // the builtin moves bits of an int
 }
 
+// base[key] += v for every lane with `on`, wave-uniform call.  Neighbouring rays mostly composite the same surfel
+// in the same step, and atomics of one instruction to one address are served one after the other, so the lanes
+// of the most frequent keys are summed across the wave and their first lane adds the total.
+__device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t key, float v) {
+    const uint32_t lane = __lane_id();
+    uint64_t rem = __ballot(on);
+#pragma unroll 1
+    for (int tries = 0; tries < 6 && rem != 0ull; ++tries) {
+        const int first = __builtin_ctzll(rem);
+        const uint32_t k0 = __builtin_amdgcn_readlane(key, first);
+        const bool same = on && key == k0;
+        const uint64_t grp = __ballot(same);
+        if (__popcll(grp) >= 3) {
+            const float s = wave_sum_f32(same ? v : 0.f);
+            if (lane == (uint32_t)first) aadd(base + k0, s);
+            on = on && !same;
+        }
+        rem &= ~grp;
+    }
+    if (on) aadd(base + key, v);
+}
+
 // Where one hit's per-surfel gradients go.  Lanes of a wave that composite the SAME surfel in the same step
 // would serialise on the same LDS addresses, so the largest groups of such lanes (found once per step) are
 // summed across the wave first and only their first lane issues the atomic; all other lanes add directly.
@@ -843,8 +865,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 Tp_hit = Tp;
                 dpt_hit = dpt;
                 Tp = Tn;
-                if (!BWD && p.training && p.a_weights != nullptr) aadd(p.a_weights + g, w);
             } while (false);
+            if (!BWD && p.training && p.a_weights != nullptr) wave_add_grouped(p.a_weights, did, (uint32_t)g, w);
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
             if (BWD && __ballot(did) != 0ull) {
                 GradSink<AUXM> sink;
