@@ -445,67 +445,8 @@ __device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t 
     if (on) aadd(base + key, v);
 }
 
-// Where one hit's per-surfel gradients go.  Lanes of a wave that composite the SAME surfel in the same step
-// would serialise on the same LDS addresses, so the largest groups of such lanes (found once per step) are
-// summed across the wave first and only their first lane issues the atomic; all other lanes add directly.
-constexpr int kBigGroups = 3;       // groups reduced across the wave per step
-constexpr int kBigGroupMin = 8;     // lanes a group needs before the reduction pays
-template <int AUXM>
-struct GradSink {
-    float *row;          // LDS row of this lane's surfel, or nullptr: write through to global memory
-    const DstParams *p;
-    uint32_t g;
-    int n_big;           // wave-uniform
-    int member;          // index of the big group this lane belongs to, or -1
-    bool lead;           // this lane issues the atomic of its big group
-    bool direct;         // this lane adds its own value (not in a big group)
-
-    // Wave-uniform: `key` is the surfel of lanes with a hit, anything for the others.
-    __device__ __forceinline__ void plan(bool did, uint32_t key) {
-        const uint32_t lane = __lane_id();
-        uint64_t rem = __ballot(did);
-        n_big = 0;
-        member = -1;
-        lead = false;
-        for (int tries = 0; tries < 2 * kBigGroups && rem != 0ull && n_big < kBigGroups; ++tries) {
-            const int first = __builtin_ctzll(rem);
-            const uint32_t k0 = __builtin_amdgcn_readlane(key, first);
-            const bool same = did && key == k0;
-            const uint64_t grp = __ballot(same);
-            if (__popcll(grp) >= kBigGroupMin) {
-                if (same) member = n_big;
-                if (lane == (uint32_t)first) lead = true;
-                ++n_big;
-            }
-            rem &= ~grp;
-        }
-        direct = did && member < 0;
-    }
-
-    // Wave-uniform call (every lane reaches it); lanes without a hit contribute nothing.
-    __device__ __forceinline__ void add(int col, float v) const {
-        float out = v;
-#pragma unroll
-        for (int k = 0; k < kBigGroups; ++k) {
-            if (k < n_big) {
-                const float s = wave_sum_f32(member == k ? v : 0.f);
-                out = (member == k) ? s : out;
-            }
-        }
-        if (direct || lead) {
-            if (row != nullptr) {
-                __hip_atomic_fetch_add(row + col, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            } else {
-                float *dst = grad_address<AUXM>(*p, g, col);
-                if (dst != nullptr) aadd(dst, out);
-            }
-        }
-    }
-};
-
-// Find or claim the table row of surfel g.
-template <int AUXM>
-__device__ __forceinline__ float *table_row(uint32_t *keys, float *rows, uint32_t g) {
+// Find or claim the table row of surfel g; -1 if none is free within a few probes.
+__device__ __forceinline__ int table_slot(uint32_t *keys, uint32_t g) {
     uint32_t slot = (g * 2654435761u) >> (32 - kTableRowsLog2);
 #pragma unroll 1
     for (int probe = 0; probe < kMaxProbe; ++probe) {
@@ -516,11 +457,102 @@ __device__ __forceinline__ float *table_row(uint32_t *keys, float *rows, uint32_
                                                  __HIP_MEMORY_SCOPE_WORKGROUP);
             k = (expected == kEmptyKey) ? g : expected;
         }
-        if (k == g) return rows + (size_t)slot * RowLayout<AUXM>::stride;
+        if (k == g) return (int)slot;
         slot = (slot + 1) & (kTableRows - 1);
     }
-    return nullptr;
+    return -1;
 }
+
+// Where one step's per-surfel gradients go.  Neighbouring rays mostly composite the same few surfels in the
+// same step, so the wave first sums the lanes of each surfel and only the sums go to the table.  That sum is
+// a matrix product: (columns x rays) times (rays x surfel groups, entries 0 or 1).  The lanes stage their
+// column values in LDS, sixteen columns at a time, and sixteen 16x16x4 fp32 MFMAs per tile produce the sums
+// of up to sixteen groups at once; lanes of further groups (rare) add their values directly.
+constexpr int kStageCols = 16;                 // columns per tile
+constexpr int kStageStride = DST_WAVE + 1;     // floats per staged column: conflict-free writes and reads
+constexpr int kStageWords = kStageCols * kStageStride;
+typedef float v4f __attribute__((ext_vector_type(4)));
+template <int AUXM>
+struct GradSink {
+    const DstParams *p;
+    float *rows;         // the block's table
+    float *stage;        // this wave's staging tile: [column in tile][lane]
+    bool did;            // this lane composited a hit in this step
+    uint32_t g;          // its surfel
+    int own_slot;        // table row of g, -1: none
+    bool stray;          // hit, but not in one of the sixteen groups
+    uint32_t members;    // bit m: the ray of lane 16*(lane/16)+m belongs to group lane%16
+    bool out_on;         // lane%16 is a group of this step
+    int out_slot;        // table row of group lane%16, -1: write through to global memory
+    uint32_t out_g;      // surfel of group lane%16
+    int limit;           // columns in use
+
+    // Wave-uniform; every lane of the wave must be active.
+    __device__ __forceinline__ void plan(uint32_t *keys) {
+        const uint32_t lane = __lane_id();
+        uint64_t rem = __ballot(did);
+        int n_groups = 0;
+        bool grouped = false;
+        uint32_t leader = 0u;
+        members = 0u;
+#pragma unroll 1
+        while (rem != 0ull && n_groups < kStageCols) {
+            const int first = __builtin_ctzll(rem);
+            const uint32_t k0 = __builtin_amdgcn_readlane(g, first);
+            const bool same = did && g == k0;
+            const uint64_t grp = __ballot(same);
+            if ((lane & 15u) == (uint32_t)n_groups) {
+                members = (uint32_t)(grp >> (lane & 48u)) & 0xFFFFu;
+                leader = (uint32_t)first;
+            }
+            grouped = grouped || same;
+            ++n_groups;
+            rem &= ~grp;
+        }
+        stray = did && !grouped;
+        out_on = (lane & 15u) < (uint32_t)n_groups;
+        own_slot = did ? table_slot(keys, g) : -1;
+        out_slot = __builtin_amdgcn_ds_bpermute((int)(leader << 2), own_slot);
+        out_g = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader << 2), (int)g);
+    }
+
+    __device__ __forceinline__ void put(int slot, uint32_t surfel, int col, float v) const {
+        if (slot >= 0) {
+            __hip_atomic_fetch_add(rows + (size_t)slot * RowLayout<AUXM>::stride + col, v, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+            float *dst = grad_address<AUXM>(*p, surfel, col);
+            if (dst != nullptr) aadd(dst, v);
+        }
+    }
+
+    // Sums of the staged tile per group, added to the groups' rows.  Wave-uniform.
+    __device__ __forceinline__ void flush(int tile) const {
+        const uint32_t lane = __lane_id();
+        const float *a = stage + (lane & 15u) * kStageStride + (lane & 48u);
+        v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < 16; ++m)
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[m], ((members >> m) & 1u) ? 1.0f : 0.0f, acc, 0, 0, 0);
+        // acc[r] = column 16*tile + 4*(lane/16) + r summed over the rays of group lane%16
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int col = tile * kStageCols + 4 * (int)(lane >> 4) + r;
+            if (out_on && col < limit && acc[r] != 0.f) put(out_slot, out_g, col, acc[r]);
+        }
+    }
+
+    // Wave-uniform calls in ascending column order (every lane reaches them); `col` is a constant after
+    // inlining.  The tile is reduced when its last column arrives; finish() reduces a partly filled last tile.
+    __device__ __forceinline__ void add(int col, float v) const {
+        stage[(col & (kStageCols - 1)) * kStageStride + __lane_id()] = did ? v : 0.f;
+        if (stray && col < limit) put(own_slot, g, col, v);
+        if ((col & (kStageCols - 1)) == kStageCols - 1) flush(col / kStageCols);
+    }
+    __device__ __forceinline__ void finish(int next_col) const {
+        if ((next_col & (kStageCols - 1)) != 0) flush(next_col / kStageCols);
+    }
+};
 
 template <int AUXM>
 struct BounceIn {  // backward: saved results of the bounce and the gradients flowing into them
@@ -547,20 +579,21 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     const float num = 1.0f - alpha;
     const float T_final = 1.0f - in.acc;
     float g_alpha = 0.f;
-    float g_col[3];
+    float g_col[3], g_aux_w[AUXM];
 #pragma unroll
     for (int ch = 0; ch < 3; ++ch) {
         g_col[ch] = in.g_rgb[ch] * w;
-        sink.add(kColColor + ch, g_col[ch]);
         g_alpha += in.g_rgb[ch] * (Tp * col[ch] - (in.rgb[ch] - run.C[ch]) / num);
         g_alpha += in.g_rgb[ch] * p.background[ch] * (-T_final / num);
     }
+#pragma unroll
+    for (int ch = 0; ch < AUXM; ++ch) g_aux_w[ch] = 0.f;
     if (p.others_precomp != nullptr) {
 #pragma unroll
         for (int ch = 0; ch < AUXM; ++ch) {
             if (ch < p.aux) {
                 float o = p.others_precomp[(size_t)p.aux * g + ch];
-                sink.add(kColAux + ch, in.g_aux[ch] * w);
+                g_aux_w[ch] = in.g_aux[ch] * w;
                 g_alpha += in.g_aux[ch] * (Tp * o - (in.aux[ch] - run.O[ch]) / num);
             }
         }
@@ -574,7 +607,6 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     g_alpha += in.g_acc * (Tp - in.acc / num);   // the reference never accumulates W (backward.cu:568)
     const float g_G = g_alpha * opac;
     const float pc = (opac * G) > 0.99f ? 0.0f : 1.0f;
-    sink.add(kColOpac, g_alpha * G * pc);
 
     // triangle that was hit, with its corner coordinates in splat units (backward.cu:583-602)
     const float *V = p.vertices + (size_t)g * 12;
@@ -616,6 +648,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     g_sy += dot(R[1], sv);
     g_mean = g_mean + (g_v1 + g_v2 + g_v3);
     // rotation: vjp of quat_rows without the normalisation Jacobian (auxiliary.h:433-477)
+    float g_rot[4];
     {
         float s = 1.0f / __builtin_sqrtf(q3 * q3 + q0 * q0 + q1 * q1 + q2 * q2);
         float w_ = q0 * s, x = q1 * s, y = q2 * s, z = q3 * s;
@@ -626,13 +659,20 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                           w_ * (gR[2].x - gR[0].z));
         float r3 = 2.f * (x * (gR[0].z + gR[2].x) + y * (gR[1].z + gR[2].y) - 2.f * z * (gR[0].x + gR[1].y) +
                           w_ * (gR[0].y - gR[1].x));
-        sink.add(kColRot + 0, r0); sink.add(kColRot + 1, r1); sink.add(kColRot + 2, r2); sink.add(kColRot + 3, r3);
+        g_rot[0] = r0; g_rot[1] = r1; g_rot[2] = r2; g_rot[3] = r3;
     }
+    // the table columns, in ascending order
+    sink.add(kColColor + 0, g_col[0]); sink.add(kColColor + 1, g_col[1]); sink.add(kColColor + 2, g_col[2]);
+    sink.add(kColOpac, g_alpha * G * pc);
     sink.add(kColScale + 0, g_sx);
     sink.add(kColScale + 1, g_sy);
+    sink.add(kColRot + 0, g_rot[0]); sink.add(kColRot + 1, g_rot[1]); sink.add(kColRot + 2, g_rot[2]); sink.add(kColRot + 3, g_rot[3]);
     sink.add(kColMean + 0, g_mean.x); sink.add(kColMean + 1, g_mean.y); sink.add(kColMean + 2, g_mean.z);
     const float hd = 0.5f * dpt;
     sink.add(kColGrad + 0, g_mean.x * hd); sink.add(kColGrad + 1, g_mean.y * hd); sink.add(kColGrad + 2, g_mean.z * hd);
+#pragma unroll
+    for (int ch = 0; ch < AUXM; ++ch) sink.add(kColAux + ch, g_aux_w[ch]);
+    if (p.colors_precomp != nullptr) sink.finish(RowLayout<AUXM>::sh0);
 
     if (p.colors_precomp == nullptr) {
         // SH backward (backward.cu:68-166); the direction gradient REPLACES the ray's (backward.cu:165)
@@ -646,32 +686,35 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
         auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
         F3 ddx = f3(0, 0, 0), ddy = f3(0, 0, 0), ddz = f3(0, 0, 0);
         const float x = rd.x, y = rd.y, z = rd.z;
-        put(0, SH0);
+        float basis[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) basis[j] = 0.f;
+        basis[0] = SH0;
         if (deg > 0) {
-            put(1, -SH1 * y);
-            put(2, SH1 * z);
-            put(3, -SH1 * x);
+            basis[1] = -SH1 * y;
+            basis[2] = SH1 * z;
+            basis[3] = -SH1 * x;
             ddx = -SH1 * S(3);
             ddy = -SH1 * S(1);
             ddz = SH1 * S(2);
             if (deg > 1) {
                 const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
-                put(4, SH2[0] * xy);
-                put(5, SH2[1] * yz);
-                put(6, SH2[2] * (2.f * zz - xx - yy));
-                put(7, SH2[3] * xz);
-                put(8, SH2[4] * (xx - yy));
+                basis[4] = SH2[0] * xy;
+                basis[5] = SH2[1] * yz;
+                basis[6] = SH2[2] * (2.f * zz - xx - yy);
+                basis[7] = SH2[3] * xz;
+                basis[8] = SH2[4] * (xx - yy);
                 ddx = ddx + SH2[0] * y * S(4) + SH2[2] * 2.f * -x * S(6) + SH2[3] * z * S(7) + SH2[4] * 2.f * x * S(8);
                 ddy = ddy + SH2[0] * x * S(4) + SH2[1] * z * S(5) + SH2[2] * 2.f * -y * S(6) + SH2[4] * 2.f * -y * S(8);
                 ddz = ddz + SH2[1] * y * S(5) + SH2[2] * 4.f * z * S(6) + SH2[3] * x * S(7);
                 if (deg > 2) {
-                    put(9, SH3[0] * y * (3.f * xx - yy));
-                    put(10, SH3[1] * xy * z);
-                    put(11, SH3[2] * y * (4.f * zz - xx - yy));
-                    put(12, SH3[3] * z * (2.f * zz - 3.f * xx - 3.f * yy));
-                    put(13, SH3[4] * x * (4.f * zz - xx - yy));
-                    put(14, SH3[5] * z * (xx - yy));
-                    put(15, SH3[6] * x * (xx - 3.f * yy));
+                    basis[9] = SH3[0] * y * (3.f * xx - yy);
+                    basis[10] = SH3[1] * xy * z;
+                    basis[11] = SH3[2] * y * (4.f * zz - xx - yy);
+                    basis[12] = SH3[3] * z * (2.f * zz - 3.f * xx - 3.f * yy);
+                    basis[13] = SH3[4] * x * (4.f * zz - xx - yy);
+                    basis[14] = SH3[5] * z * (xx - yy);
+                    basis[15] = SH3[6] * x * (xx - 3.f * yy);
                     ddx = ddx + (SH3[0] * 6.f * xy) * S(9) + (SH3[1] * yz) * S(10) + (SH3[2] * -2.f * xy) * S(11) +
                           (SH3[3] * -6.f * xz) * S(12) + (SH3[4] * (-3.f * xx + 4.f * zz - yy)) * S(13) +
                           (SH3[5] * 2.f * xz) * S(14) + (SH3[6] * 3.f * (xx - yy)) * S(15);
@@ -684,6 +727,9 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                 }
             }
         }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) put(j, basis[j]);
+        sink.finish(RowLayout<AUXM>::cols);
         if (did) g_rd = f3(dot(ddx, gc), dot(ddy, gc), dot(ddz, gc));
     }
 }
@@ -740,8 +786,8 @@ template <bool BWD, int AUXM, bool REC>
 __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
-                                            uint32_t &n_con, uint32_t *tab_keys, float *tab_rows, const RecView &rv,
-                                            int bounce
+                                            uint32_t &n_con, uint32_t *tab_keys, float *tab_rows, float *stage,
+                                            const RecView &rv, int bounce
 #ifdef DST_STATS
                                             , WaveStats &ws
 #endif
@@ -870,10 +916,13 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
             if (BWD && __ballot(did) != 0ull) {
                 GradSink<AUXM> sink;
-                sink.plan(did, did ? (uint32_t)g : 0xFFFFFFFFu);
-                sink.row = did ? table_row<AUXM>(tab_keys, tab_rows, (uint32_t)g) : nullptr;
                 sink.p = &p;
+                sink.rows = tab_rows;
+                sink.stage = stage;
+                sink.did = did;
                 sink.g = (uint32_t)g;
+                sink.limit = (p.colors_precomp == nullptr) ? RowLayout<AUXM>::cols : RowLayout<AUXM>::sh0;
+                sink.plan(tab_keys);
                 hit_backward<AUXM>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
                                    q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did);
             }
@@ -925,6 +974,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     // is what the block's gradient table and the caches live on
     __shared__ uint32_t s_keys[BWD ? kTableRows : 1];
     __shared__ float s_rows[BWD ? kTableRows * RowLayout<AUXM>::stride : 1];
+    __shared__ float s_stage[BWD ? kWavesPerBlock * kStageWords : 1];
     uint32_t *tab_keys = s_keys;
     float *tab_rows = s_rows;
     if (BWD) {
@@ -980,7 +1030,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, rv, i WS_ARG);
+            walk_bounce<false, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -1120,7 +1170,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, rv, i WS_ARG);
+            walk_bounce<true, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
         }
         if (inside) {
             p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
