@@ -22,6 +22,10 @@ constexpr float kStartOffset = 0.06f;
 constexpr float kNear = 0.2f;
 constexpr float kTmin = 0.0001f;
 constexpr int kWavesPerBlock = 4;
+#ifndef DST_FWD_WPB
+#define DST_FWD_WPB 1
+#endif
+constexpr int kFwdWavesPerBlock = DST_FWD_WPB;   // 1 or kWavesPerBlock
 
 __device__ const float SH0 = 0.28209479177387814f;
 __device__ const float SH1 = 0.4886025119029199f;
@@ -983,15 +987,21 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             s_rows[k] = 0.f;
         __syncthreads();
     }
-    const uint32_t wv = threadIdx.x / DST_WAVE;
+    // Backward: a block is the four waves of a 16x16 pixel tile (they share the gradient table).  Forward: the
+    // waves share nothing, so each is a workgroup of its own and takes a free wave slot as soon as there is
+    // one; workgroups x, x+8, x+16, x+24 (same XCD under round-robin dispatch) are the four waves of a tile.
+    uint32_t bid = blockIdx.x, wv = threadIdx.x / DST_WAVE;
+    if (!BWD && kFwdWavesPerBlock == 1) {
+        bid = (blockIdx.x >> 5) * 8u + (blockIdx.x & 7u);
+        wv = (blockIdx.x >> 3) & 3u;
+    }
     // Blocks keep the dispatch order (row-major over the 16x16 pixel tiles).  Re-numbering them so that each of
     // the 8 XCDs owns a band or whole rows of the image was measured and is slower on the 1080p room scene
     // (+15 % / +8 % forward): the chip then works on 8 distant image regions at once and the shared last-level
     // cache sees 8 times more distinct BVH data, which costs more than the per-XCD L2 gains.
-    const uint32_t bid = blockIdx.x;
     RecView rv = {nullptr, nullptr, nullptr, 0u};
     if (REC) {
-        const uint32_t n_waves = gridDim.x * kWavesPerBlock, slots_ = (uint32_t)p.mtd_alloc + 1u;
+        const uint32_t n_waves = btiles_x * ((tiles_y + 1u) / 2u) * kWavesPerBlock, slots_ = (uint32_t)p.mtd_alloc + 1u;
         const uint64_t dir_words = ((uint64_t)n_waves * slots_ + 1u) / 2u;
         rv.base = p.hit_record;
         rv.dir = reinterpret_cast<uint32_t *>(p.hit_record + 2) + (size_t)(bid * kWavesPerBlock + wv) * slots_;
@@ -1201,7 +1211,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
 #define DST_BWD_WAVES 3
 #endif
 template <int AUXM, bool REC>
-__global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
+__global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x) {
     trace_body<false, AUXM, REC>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
@@ -1234,6 +1244,10 @@ TileGrid tile_grid(int H, int W) {
 template <bool BWD, bool REC>
 void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipStream_t stream) {
     dim3 grid(t.btiles_x * t.btiles_y), block(kWavesPerBlock * DST_WAVE);
+    if (!BWD && kFwdWavesPerBlock == 1) {
+        grid = dim3((t.btiles_x * t.btiles_y + 7u) / 8u * 32u);
+        block = dim3(DST_WAVE);
+    }
 #define DST_LAUNCH(AUX)                                                                                            \
     do {                                                                                                           \
         if (BWD)                                                                                                   \
