@@ -11,7 +11,9 @@
 #define DST_NO_PARENT 0xFFFFFFFFu
 #define DST_WAVE 64
 
-#define DST_GROUP 2            // quads per leaf group (a subtree of at most this many leaves is tested as a unit)
+#ifndef DST_GROUP
+#define DST_GROUP 2             // quads per leaf group (a subtree of at most this many leaves is tested as a unit)
+#endif
 #define DST_WIDE 4             // children per traversal node
 #define DST_REF_FIRST_MASK 0x0FFFFFFFu   // leaf-group reference: DST_LEAF_BIT | (count-1) << 28 | first leaf position
 #define DST_MAX_SURFELS 0x0FFFFFFFu

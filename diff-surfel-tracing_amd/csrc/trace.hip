@@ -229,7 +229,7 @@ __device__ __forceinline__ void kbuf_insert(KBuf &b, uint64_t x, bool on) {
 }
 
 #ifdef DST_STATS
-struct WaveStats { unsigned long long nodes, leaves, t_trav, t_comp, chunks, leaf_any; };
+struct WaveStats { unsigned long long nodes, leaves, t_trav, t_comp, chunks, leaf_any, t_plan, t_hb, steps; };
 #define STAT(x) x
 #else
 #define STAT(x)
@@ -383,8 +383,6 @@ __device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v);
 #ifndef DST_TABLE_ROWS_LOG2
 #define DST_TABLE_ROWS_LOG2 7
 #endif
-constexpr int kTableRowsLog2 = DST_TABLE_ROWS_LOG2;
-constexpr int kTableRows = 1 << kTableRowsLog2;
 constexpr uint32_t kEmptyKey = 0xFFFFFFFFu;
 constexpr int kMaxProbe = 8;
 // row columns: colour 0-2, opacity 3, scales 4-5, rotation 6-9, mean 10-12, densification mean 13-15,
@@ -394,6 +392,9 @@ template <int AUXM> struct RowLayout {
     static constexpr int sh0 = kColAux + AUXM;
     static constexpr int cols = sh0 + 48;
     static constexpr int stride = cols | 1;     // odd: rows spread over all LDS banks
+    // rows of the block's table: with more auxiliary channels the rows are longer, and three blocks must fit a CU
+    static constexpr int rows_log2 = AUXM <= 2 ? DST_TABLE_ROWS_LOG2 : DST_TABLE_ROWS_LOG2 - 1;
+    static constexpr int rows = 1 << rows_log2;
 };
 
 // Address in the caller's gradient tensors of column `col` of surfel g (nullptr: nothing to write).
@@ -450,8 +451,9 @@ __device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t 
 }
 
 // Find or claim the table row of surfel g; -1 if none is free within a few probes.
+template <int ROWS_LOG2>
 __device__ __forceinline__ int table_slot(uint32_t *keys, uint32_t g) {
-    uint32_t slot = (g * 2654435761u) >> (32 - kTableRowsLog2);
+    uint32_t slot = (g * 2654435761u) >> (32 - ROWS_LOG2);
 #pragma unroll 1
     for (int probe = 0; probe < kMaxProbe; ++probe) {
         uint32_t k = __hip_atomic_load(keys + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -462,7 +464,7 @@ __device__ __forceinline__ int table_slot(uint32_t *keys, uint32_t g) {
             k = (expected == kEmptyKey) ? g : expected;
         }
         if (k == g) return (int)slot;
-        slot = (slot + 1) & (kTableRows - 1);
+        slot = (slot + 1) & ((1u << ROWS_LOG2) - 1u);
     }
     return -1;
 }
@@ -515,7 +517,7 @@ struct GradSink {
         }
         stray = did && !grouped;
         out_on = (lane & 15u) < (uint32_t)n_groups;
-        own_slot = did ? table_slot(keys, g) : -1;
+        own_slot = did ? table_slot<RowLayout<AUXM>::rows_log2>(keys, g) : -1;
         out_slot = __builtin_amdgcn_ds_bpermute((int)(leader << 2), own_slot);
         out_g = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader << 2), (int)g);
     }
@@ -580,15 +582,16 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                                              const float *__restrict__ sh, F3 &g_ro, F3 &g_rd,
                                              const GradSink<AUXM> &sink, bool did) {
 #pragma clang fp contract(fast)
-    const float num = 1.0f - alpha;
+    // gradient algebra only: divisions become multiplications by a hardware reciprocal (1 ulp)
+    const float num = 1.0f - alpha, inv_num = __builtin_amdgcn_rcpf(num);
     const float T_final = 1.0f - in.acc;
     float g_alpha = 0.f;
     float g_col[3], g_aux_w[AUXM];
 #pragma unroll
     for (int ch = 0; ch < 3; ++ch) {
         g_col[ch] = in.g_rgb[ch] * w;
-        g_alpha += in.g_rgb[ch] * (Tp * col[ch] - (in.rgb[ch] - run.C[ch]) / num);
-        g_alpha += in.g_rgb[ch] * p.background[ch] * (-T_final / num);
+        g_alpha += in.g_rgb[ch] * (Tp * col[ch] - (in.rgb[ch] - run.C[ch]) * inv_num);
+        g_alpha += in.g_rgb[ch] * p.background[ch] * (-T_final * inv_num);
     }
 #pragma unroll
     for (int ch = 0; ch < AUXM; ++ch) g_aux_w[ch] = 0.f;
@@ -598,17 +601,17 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
             if (ch < p.aux) {
                 float o = p.others_precomp[(size_t)p.aux * g + ch];
                 g_aux_w[ch] = in.g_aux[ch] * w;
-                g_alpha += in.g_aux[ch] * (Tp * o - (in.aux[ch] - run.O[ch]) / num);
+                g_alpha += in.g_aux[ch] * (Tp * o - (in.aux[ch] - run.O[ch]) * inv_num);
             }
         }
     }
     const float g_D = in.g_dpt * w;
-    g_alpha += in.g_dpt * (Tp * dpt - (in.dpt - run.D) / num);
+    g_alpha += in.g_dpt * (Tp * dpt - (in.dpt - run.D) * inv_num);
     const F3 g_N = f3(in.g_nrm[0] * w, in.g_nrm[1] * w, in.g_nrm[2] * w);
-    g_alpha += in.g_nrm[0] * (Tp * normal.x - (in.nrm[0] - run.N[0]) / num) +
-               in.g_nrm[1] * (Tp * normal.y - (in.nrm[1] - run.N[1]) / num) +
-               in.g_nrm[2] * (Tp * normal.z - (in.nrm[2] - run.N[2]) / num);
-    g_alpha += in.g_acc * (Tp - in.acc / num);   // the reference never accumulates W (backward.cu:568)
+    g_alpha += in.g_nrm[0] * (Tp * normal.x - (in.nrm[0] - run.N[0]) * inv_num) +
+               in.g_nrm[1] * (Tp * normal.y - (in.nrm[1] - run.N[1]) * inv_num) +
+               in.g_nrm[2] * (Tp * normal.z - (in.nrm[2] - run.N[2]) * inv_num);
+    g_alpha += in.g_acc * (Tp - in.acc * inv_num);   // the reference never accumulates W (backward.cu:568)
     const float g_G = g_alpha * opac;
     const float pc = (opac * G) > 0.99f ? 0.0f : 1.0f;
 
@@ -626,23 +629,24 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     const float gu = k * -G * u, gv = k * -G * v;
     F3 gR[3];
     const F3 rel = xyz - mean;
-    gR[0] = gu * rel / sx;
-    gR[1] = gv * rel / sy;
+    const float inv_sx = __builtin_amdgcn_rcpf(sx), inv_sy = __builtin_amdgcn_rcpf(sy);
+    gR[0] = (gu * inv_sx) * rel;
+    gR[1] = (gv * inv_sy) * rel;
     gR[2] = g_N * nsign;
-    float g_sx = k * (G * u * u / sx), g_sy = k * (G * v * v / sy);
-    F3 g_mean = k * (G * (R[0] * u / sx + R[1] * v / sy));
-    const F3 g_xyz = (gu / sx) * R[0] + (gv / sy) * R[1];
+    float g_sx = k * (G * u * u * inv_sx), g_sy = k * (G * v * v * inv_sy);
+    F3 g_mean = k * (G * (R[0] * (u * inv_sx) + R[1] * (v * inv_sy)));
+    const F3 g_xyz = (gu * inv_sx) * R[0] + (gv * inv_sy) * R[1];
     const float g_d = g_D + dot(g_xyz, rd);
     const F3 n = cross(v2 - v1, v3 - v1);
     const F3 c = v1 - ro;
-    const float pp = dot(n, c), q = dot(n, rd);
-    const F3 g_n = (c - (pp / q) * rd) / q;
-    const F3 g_v1 = g_d * cross(v2 - v3, g_n) + g_d * n / q;
+    const float pp = dot(n, c), q = dot(n, rd), inv_q = __builtin_amdgcn_rcpf(q);
+    const F3 g_n = (c - (pp * inv_q) * rd) * inv_q;
+    const F3 g_v1 = g_d * cross(v2 - v3, g_n) + (g_d * inv_q) * n;
     const F3 g_v2 = g_d * cross(v3 - v1, g_n);
     const F3 g_v3 = g_d * cross(v1 - v2, g_n);
     if (did) {
-        g_ro = g_ro + (g_xyz + (g_d * -n) / q);
-        g_rd = g_rd + (g_xyz * dpt + ((g_d * -pp) / (q * q)) * n);
+        g_ro = g_ro + (g_xyz + (-g_d * inv_q) * n);
+        g_rd = g_rd + (g_xyz * dpt + ((g_d * -pp) * (inv_q * inv_q)) * n);
     }
     const F3 su = h1.x * g_v1 + h2.x * g_v2 + h3.x * g_v3;
     const F3 sv = h1.y * g_v1 + h2.y * g_v2 + h3.y * g_v3;
@@ -654,7 +658,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     // rotation: vjp of quat_rows without the normalisation Jacobian (auxiliary.h:433-477)
     float g_rot[4];
     {
-        float s = 1.0f / __builtin_sqrtf(q3 * q3 + q0 * q0 + q1 * q1 + q2 * q2);
+        float s = __builtin_amdgcn_rsqf(q3 * q3 + q0 * q0 + q1 * q1 + q2 * q2);
         float w_ = q0 * s, x = q1 * s, y = q2 * s, z = q3 * s;
         float r0 = 2.f * (x * (gR[1].z - gR[2].y) + y * (gR[2].x - gR[0].z) + z * (gR[0].y - gR[1].x));
         float r1 = 2.f * (-2.f * x * (gR[1].y + gR[2].z) + y * (gR[0].y + gR[1].x) + z * (gR[0].z + gR[2].x) +
@@ -926,9 +930,12 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 sink.did = did;
                 sink.g = (uint32_t)g;
                 sink.limit = (p.colors_precomp == nullptr) ? RowLayout<AUXM>::cols : RowLayout<AUXM>::sh0;
+                STAT(unsigned long long d0 = __builtin_readcyclecounter();)
                 sink.plan(tab_keys);
+                STAT(unsigned long long d1 = __builtin_readcyclecounter(); ws.t_plan += d1 - d0; ws.steps++;)
                 hit_backward<AUXM>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
                                    q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did);
+                STAT(ws.t_hb += __builtin_readcyclecounter() - d1;)
             }
         }
         STAT(ws.t_comp += __builtin_readcyclecounter() - c1;)
@@ -976,6 +983,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
+    constexpr int kTableRows = RowLayout<AUXM>::rows;
     __shared__ uint32_t s_keys[BWD ? kTableRows : 1];
     __shared__ float s_rows[BWD ? kTableRows * RowLayout<AUXM>::stride : 1];
     __shared__ float s_stage[BWD ? kWavesPerBlock * kStageWords : 1];
@@ -1023,7 +1031,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     const F3 ray_o = ld3(p.ray_o + 3 * r), ray_d = ld3(p.ray_d + 3 * r);
     uint32_t n_proc = 0, n_con = 0;
 #ifdef DST_STATS
-    WaveStats ws = {0, 0, 0, 0, 0, 0};
+    WaveStats ws = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 #define WS_ARG , ws
 #else
 #define WS_ARG
@@ -1182,6 +1190,16 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             walk_bounce<true, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
         }
+#ifdef DST_STATS   // development build only: counters must then hold 8 entries
+        if (p.counters != nullptr && lane == 0) {
+            atomicAdd(p.counters + 2, ws.steps);
+            atomicAdd(p.counters + 3, ws.t_plan);
+            atomicAdd(p.counters + 4, ws.t_trav);
+            atomicAdd(p.counters + 5, ws.t_comp);
+            atomicAdd(p.counters + 6, ws.chunks);
+            atomicAdd(p.counters + 7, ws.t_hb);
+        }
+#endif
         if (inside) {
             p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
             p.dL_dray_d[3 * r + 0] = g_rd.x; p.dL_dray_d[3 * r + 1] = g_rd.y; p.dL_dray_d[3 * r + 2] = g_rd.z;

@@ -244,7 +244,7 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
                            transMat_precomp, viewmatrix, projmatrix, campos, prefiltered, debug, max_trace_depth,
                            specular_threshold, out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val,
                            dL_dout_rgb, dL_dout_dpt, dL_dout_acc, dL_dout_norm, dL_dout_dist, dL_dout_aux,
-                           events=None, hit_record=None):
+                           events=None, hit_record=None, counters=None):
     """Reference TraceSurfelsBackwardCUDA (trace_surfels.cpp:307-464): returns (dL_dray_o, dL_dray_d, dL_dmeans3D,
     dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers, dL_dopacities, dL_dscales, dL_drotations,
     dL_dtransMat_precomp)."""
@@ -286,6 +286,7 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
         ctx.record_blocks_per_wave = max(ctx.record_blocks_per_wave, 1.25 * asked / hit_record.n_waves)
         if asked <= hit_record.blocks:
             p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
+    p.counters = _ptr(counters)
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))
