@@ -45,8 +45,10 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="config3", choices=["config1", "config2", "config3"])
-    ap.add_argument("--cpu-stride", type=int, default=2, help="CPU baseline traces every n-th pixel row and column")
+    ap.add_argument("--cpu-stride", type=int, default=1, help="CPU baseline traces every n-th pixel row and column")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run one plain 1 GiB read + 1 GiB write kernel (a yardstick for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (rays would be sharded across "
@@ -105,6 +107,12 @@ def main():
 
     for _ in range(args.warmup):
         step()
+    if args.traffic_probe:
+        probe_src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        probe_dst = torch.empty_like(probe_src)
+        torch.mul(probe_src, 2.0, out=probe_dst)   # reads 2^30 bytes, writes 2^30 bytes
+        torch.cuda.synchronize()
+        del probe_src, probe_dst
     step(count=True)
     torch.cuda.synchronize()
     n_proc, n_con = counters.tolist()
