@@ -36,6 +36,8 @@ __device__ const float SH3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.45
                                  -0.5900435899266435f};
 
 struct F3 { float x, y, z; };
+// Lanes for which `b` holds (the compare result itself becomes the mask: no 0/1 detour through a register).
+__device__ __forceinline__ uint64_t wave_ballot(bool b) { return __builtin_amdgcn_ballot_w64(b); }
 __device__ __forceinline__ F3 f3(float x, float y, float z) { return F3{x, y, z}; }
 __device__ __forceinline__ F3 operator+(F3 a, F3 b) { return F3{a.x + b.x, a.y + b.y, a.z + b.z}; }
 __device__ __forceinline__ F3 operator-(F3 a, F3 b) { return F3{a.x - b.x, a.y - b.y, a.z - b.z}; }
@@ -188,15 +190,16 @@ struct RaySlabFast {
     float cnx, cny, cnz;   // -o/d - widening: added to (near face)/d
     float cfx, cfy, cfz;   // -o/d + widening: added to (far face)/d
 };
-__device__ __forceinline__ bool slab_hit_fast(const RaySlabFast &s, float nx, float ny, float nz, float fx, float fy,
-                                              float fz, float tmax, float &tn) {
+// Returns the lanes that hit as a mask (the compare writes the wave mask directly).
+__device__ __forceinline__ uint64_t slab_hit_fast(const RaySlabFast &s, float nx, float ny, float nz, float fx,
+                                                  float fy, float fz, float tmax, float &tn) {
     const float a = __builtin_fmaf(nx, s.ix, s.cnx), b = __builtin_fmaf(ny, s.iy, s.cny),
                 c = __builtin_fmaf(nz, s.iz, s.cnz);
     const float e = __builtin_fmaf(fx, s.ix, s.cfx), f = __builtin_fmaf(fy, s.iy, s.cfy),
                 g = __builtin_fmaf(fz, s.iz, s.cfz);
     tn = __builtin_fmaxf(__builtin_fmaxf(a, b), __builtin_fmaxf(c, 0.0f));
     const float tf = __builtin_fminf(__builtin_fminf(e, f), __builtin_fminf(g, tmax));
-    return tn <= tf;
+    return __builtin_amdgcn_fcmpf(tn, tf, 5);   // 5 = ordered <=
 }
 
 // The 16 nearest hits of a lane, ascending.  One entry = (bits of t) << 32 | idx: t is positive, so the
@@ -251,7 +254,7 @@ __device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool 
 #undef LF3
     const uint64_t x = kb_pack(t, 2u * L[18] + tri);
     const bool adm = hit && (x < buf.e[kChunk - 1]);
-    if (__ballot(adm) != 0ull) {
+    if (wave_ballot(adm) != 0ull) {
         STAT(ws.leaf_any++;)
         cnt += adm ? 1u : 0u;
         kbuf_insert(buf, x, adm);
@@ -308,17 +311,18 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
 #pragma unroll
                 for (int k = 0; k < DST_WIDE; ++k) {
                     float tn;
-                    const bool h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
-                                                 __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
-                                                 __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn) &&
-                                   (uint32_t)k < n_child;   // unused slots are never entered
-                    const bool any = __ballot(h) != 0ull;
-                    // entry distance of the representative lane (non-negative, so its bits order like the value)
-                    const uint32_t kk = __builtin_amdgcn_readlane(h ? __float_as_uint(tn) : 0x7F800000u, rep);
-                    key[k] = any ? kk : 0xFFFFFFFFu;
+                    const uint64_t h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
+                                                     __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
+                                                     __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn);
+                    // Key: entry distance of the representative lane if it hits the child itself (non-negative,
+                    // so its bits order like the value), +inf if only other lanes do, all ones if nobody does or
+                    // the slot is unused.
+                    const uint32_t kk = __builtin_amdgcn_readlane(__float_as_uint(tn), rep);
+                    const uint32_t mine = ((h >> rep) & 1ull) ? kk : 0x7F800000u;
+                    key[k] = ((uint32_t)k < n_child && h != 0ull) ? mine : 0xFFFFFFFFu;
                     cref[k] = tail[k];
-                    n_push += any ? 1 : 0;
                 }
+                n_push = 4 - (int)((key[0] >> 31) + (key[1] >> 31) + (key[2] >> 31) + (key[3] >> 31));
             }
             if (n_push > 0) {
                 // sort the four (key, ref) pairs, nearest first; children nobody wants carry the largest key
@@ -356,7 +360,7 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
                                            , WaveStats &ws
 #endif
 ) {
-    const uint64_t live = __ballot(active);
+    const uint64_t live = wave_ballot(active);
     if (live == 0ull) return;
     const RaySlab slab = make_slab(o, d, max_abs);
     // The walk assumes one set of direction signs per packet (the near face of every box is then the same for
@@ -368,7 +372,7 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
         const int rep = __builtin_ctzll(todo);   // also the lane whose entry distances order the children
         const uint32_t sgn = __builtin_amdgcn_readlane(my_sgn, rep);
         const bool mine = active && my_sgn == sgn;
-        todo &= ~__ballot(mine);
+        todo &= ~wave_ballot(mine);
         packet_walk(acc, slab, sgn, o, d, mine, rep, buf, cnt WSP);
     }
 }
@@ -433,13 +437,13 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
 // of the most frequent keys are summed across the wave and their first lane adds the total.
 __device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t key, float v) {
     const uint32_t lane = __lane_id();
-    uint64_t rem = __ballot(on);
+    uint64_t rem = wave_ballot(on);
 #pragma unroll 1
     for (int tries = 0; tries < 6 && rem != 0ull; ++tries) {
         const int first = __builtin_ctzll(rem);
         const uint32_t k0 = __builtin_amdgcn_readlane(key, first);
         const bool same = on && key == k0;
-        const uint64_t grp = __ballot(same);
+        const uint64_t grp = wave_ballot(same);
         if (__popcll(grp) >= 3) {
             const float s = wave_sum_f32(same ? v : 0.f);
             if (lane == (uint32_t)first) aadd(base + k0, s);
@@ -487,6 +491,7 @@ struct GradSink {
     uint32_t g;          // its surfel
     int own_slot;        // table row of g, -1: none
     bool stray;          // hit, but not in one of the sixteen groups
+    bool any_stray;      // wave-uniform: some lane is a stray
     uint32_t members;    // bit m: the ray of lane 16*(lane/16)+m belongs to group lane%16
     bool out_on;         // lane%16 is a group of this step
     int out_slot;        // table row of group lane%16, -1: write through to global memory
@@ -496,7 +501,7 @@ struct GradSink {
     // Wave-uniform; every lane of the wave must be active.
     __device__ __forceinline__ void plan(uint32_t *keys) {
         const uint32_t lane = __lane_id();
-        uint64_t rem = __ballot(did);
+        uint64_t rem = wave_ballot(did);
         int n_groups = 0;
         bool grouped = false;
         uint32_t leader = 0u;
@@ -506,7 +511,7 @@ struct GradSink {
             const int first = __builtin_ctzll(rem);
             const uint32_t k0 = __builtin_amdgcn_readlane(g, first);
             const bool same = did && g == k0;
-            const uint64_t grp = __ballot(same);
+            const uint64_t grp = wave_ballot(same);
             if ((lane & 15u) == (uint32_t)n_groups) {
                 members = (uint32_t)(grp >> (lane & 48u)) & 0xFFFFu;
                 leader = (uint32_t)first;
@@ -516,6 +521,7 @@ struct GradSink {
             rem &= ~grp;
         }
         stray = did && !grouped;
+        any_stray = wave_ballot(stray) != 0ull;
         out_on = (lane & 15u) < (uint32_t)n_groups;
         own_slot = did ? table_slot<RowLayout<AUXM>::rows_log2>(keys, g) : -1;
         out_slot = __builtin_amdgcn_ds_bpermute((int)(leader << 2), own_slot);
@@ -552,7 +558,9 @@ struct GradSink {
     // inlining.  The tile is reduced when its last column arrives; finish() reduces a partly filled last tile.
     __device__ __forceinline__ void add(int col, float v) const {
         stage[(col & (kStageCols - 1)) * kStageStride + __lane_id()] = did ? v : 0.f;
-        if (stray && col < limit) put(own_slot, g, col, v);
+        if (any_stray) {   // rare: more than sixteen surfels in one step
+            if (stray && col < limit) put(own_slot, g, col, v);
+        }
         if ((col & (kStageCols - 1)) == kStageCols - 1) flush(col / kStageCols);
     }
     __device__ __forceinline__ void finish(int next_col) const {
@@ -811,7 +819,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     bool live = lane_on;
     KBuf buf;
     uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
-    while (__ballot(live) != 0ull) {
+    while (wave_ballot(live) != 0ull) {
         uint32_t cnt = 0;
         STAT(ws.chunks++; unsigned long long c0 = __builtin_readcyclecounter();)
         // Where the compositing loop below takes its entries from: the recorded block, one slot at a time
@@ -832,7 +840,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
 #pragma unroll 1
         for (int it = 0; it < kChunk; ++it) {
             const bool on = live && !stop && (uint32_t)it < cnt;
-            if (__ballot(on) == 0ull) break;
+            if (wave_ballot(on) == 0ull) break;
             // next entry in depth order (consumed slots need no reset: the buffer is rebuilt for every chunk)
             uint64_t e;
             if (REC && BWD) {
@@ -922,7 +930,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             } while (false);
             if (!BWD && p.training && p.a_weights != nullptr) wave_add_grouped(p.a_weights, did, (uint32_t)g, w);
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
-            if (BWD && __ballot(did) != 0ull) {
+            if (BWD && wave_ballot(did) != 0ull) {
                 GradSink<AUXM> sink;
                 sink.p = &p;
                 sink.rows = tab_rows;
