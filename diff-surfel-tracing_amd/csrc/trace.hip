@@ -454,7 +454,8 @@ __device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t 
     if (on) aadd(base + key, v);
 }
 
-// Find or claim the table row of surfel g; -1 if none is free within a few probes.
+// Find or claim the table row of surfel g; -1 if none is free within a few probes.  keys[rows] counts the
+// rows claimed since the table was last emptied.
 template <int ROWS_LOG2>
 __device__ __forceinline__ int table_slot(uint32_t *keys, uint32_t g) {
     uint32_t slot = (g * 2654435761u) >> (32 - ROWS_LOG2);
@@ -465,7 +466,12 @@ __device__ __forceinline__ int table_slot(uint32_t *keys, uint32_t g) {
             uint32_t expected = kEmptyKey;
             __hip_atomic_compare_exchange_strong(keys + slot, &expected, g, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                                  __HIP_MEMORY_SCOPE_WORKGROUP);
-            k = (expected == kEmptyKey) ? g : expected;
+            if (expected == kEmptyKey) {
+                k = g;
+                __hip_atomic_fetch_add(keys + (1u << ROWS_LOG2), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+                k = expected;
+            }
         }
         if (k == g) return (int)slot;
         slot = (slot + 1) & ((1u << ROWS_LOG2) - 1u);
@@ -796,6 +802,29 @@ __device__ __forceinline__ const uint64_t *rec_open(const RecView &rv, uint32_t 
     return b;
 }
 
+// Block-wide: write the table to the caller's gradient tensors and empty it.  Consecutive threads take
+// consecutive columns of a row, so the 48 SH columns of a surfel go out as contiguous atomics.  The caller
+// puts barriers around it.
+template <int AUXM>
+__device__ __forceinline__ void table_flush(const DstParams &p, uint32_t *keys, float *rows) {
+    constexpr int stride = RowLayout<AUXM>::stride, n_rows = RowLayout<AUXM>::rows;
+    for (int k = threadIdx.x; k < n_rows * stride; k += kWavesPerBlock * DST_WAVE) {
+        const int row = k / stride, col = k - row * stride;
+        const uint32_t g = keys[row];
+        if (g == kEmptyKey || col >= RowLayout<AUXM>::cols) continue;
+        const float v = rows[k];
+        if (v == 0.f) continue;
+        rows[k] = 0.f;
+        float *dst = grad_address<AUXM>(p, g, col);
+        if (dst != nullptr) aadd(dst, v);
+    }
+}
+template <int AUXM>
+__device__ __forceinline__ void table_clear_keys(uint32_t *keys) {
+    for (int k = threadIdx.x; k <= RowLayout<AUXM>::rows; k += kWavesPerBlock * DST_WAVE)
+        keys[k] = (k < RowLayout<AUXM>::rows) ? kEmptyKey : 0u;
+}
+
 // One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
 // and for BWD the per-hit gradients of the re-trace (reference backward.cu:332-655).
 template <bool BWD, int AUXM, bool REC>
@@ -819,7 +848,16 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     bool live = lane_on;
     KBuf buf;
     uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
-    while (wave_ballot(live) != 0ull) {
+    for (;;) {
+        // Backward: the four waves of the block take their chunks in step, so that between two rounds nobody
+        // touches the gradient table and it can be emptied when it fills up.
+        const bool wave_live = wave_ballot(live) != 0ull;
+        if (BWD) {
+            if (__syncthreads_or(wave_live ? 1 : 0) == 0) break;
+        } else if (!wave_live) {
+            break;
+        }
+        if (wave_live) do {
         uint32_t cnt = 0;
         STAT(ws.chunks++; unsigned long long c0 = __builtin_readcyclecounter();)
         // Where the compositing loop below takes its entries from: the recorded block, one slot at a time
@@ -828,7 +866,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         const uint32_t lane_ = __lane_id();
         if (REC && BWD) {
             rec_block = rec_open(rv, rec_pos, cnt);
-            if (rec_block == nullptr) break;   // cannot happen with a complete record
+            if (rec_block == nullptr) { live = false; break; }   // cannot happen with a complete record
         } else {
             kbuf_reset(buf);
             packet_knn(acc, max_abs, ot, rd, live, buf, cnt WSP);
@@ -940,7 +978,9 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 sink.limit = (p.colors_precomp == nullptr) ? RowLayout<AUXM>::cols : RowLayout<AUXM>::sh0;
                 STAT(unsigned long long d0 = __builtin_readcyclecounter();)
                 sink.plan(tab_keys);
-                STAT(unsigned long long d1 = __builtin_readcyclecounter(); ws.t_plan += d1 - d0; ws.steps++;)
+                STAT(unsigned long long d1 = __builtin_readcyclecounter(); ws.t_plan += d1 - d0; ws.steps++;
+                     ws.nodes += __popcll(wave_ballot(did && sink.own_slot < 0)); ws.leaves += __popcll(wave_ballot(sink.stray));
+                     ws.leaf_any += __popcll(wave_ballot(did));)
                 hit_backward<AUXM>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
                                    q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did);
                 STAT(ws.t_hb += __builtin_readcyclecounter() - d1;)
@@ -956,6 +996,15 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             } else {
                 pay_dpt = next_dpt;
                 ot = f3(ro.x + pay_dpt * rd.x, ro.y + pay_dpt * rd.y, ro.z + pay_dpt * rd.z);
+            }
+        }
+        } while (false);
+        if (BWD) {
+            __syncthreads();   // every wave's additions of this round are in the table
+            if (tab_keys[RowLayout<AUXM>::rows] > (uint32_t)(3 * RowLayout<AUXM>::rows / 4)) {
+                table_flush<AUXM>(p, tab_keys, tab_rows);
+                __syncthreads();
+                table_clear_keys<AUXM>(tab_keys);   // the barrier at the top of the next round publishes it
             }
         }
     }
@@ -992,13 +1041,13 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     constexpr int kTableRows = RowLayout<AUXM>::rows;
-    __shared__ uint32_t s_keys[BWD ? kTableRows : 1];
+    __shared__ uint32_t s_keys[BWD ? kTableRows + 1 : 1];   // + the count of claimed rows
     __shared__ float s_rows[BWD ? kTableRows * RowLayout<AUXM>::stride : 1];
     __shared__ float s_stage[BWD ? kWavesPerBlock * kStageWords : 1];
     uint32_t *tab_keys = s_keys;
     float *tab_rows = s_rows;
     if (BWD) {
-        for (int k = threadIdx.x; k < kTableRows; k += kWavesPerBlock * DST_WAVE) s_keys[k] = kEmptyKey;
+        table_clear_keys<AUXM>(s_keys);
         for (int k = threadIdx.x; k < kTableRows * RowLayout<AUXM>::stride; k += kWavesPerBlock * DST_WAVE)
             s_rows[k] = 0.f;
         __syncthreads();
@@ -1198,7 +1247,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             walk_bounce<true, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
         }
-#ifdef DST_STATS   // development build only: counters must then hold 8 entries
+#ifdef DST_STATS   // development build only: counters must then hold 11 entries
         if (p.counters != nullptr && lane == 0) {
             atomicAdd(p.counters + 2, ws.steps);
             atomicAdd(p.counters + 3, ws.t_plan);
@@ -1206,25 +1255,17 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             atomicAdd(p.counters + 5, ws.t_comp);
             atomicAdd(p.counters + 6, ws.chunks);
             atomicAdd(p.counters + 7, ws.t_hb);
+            atomicAdd(p.counters + 8, ws.nodes);
+            atomicAdd(p.counters + 9, ws.leaves);
+            atomicAdd(p.counters + 10, ws.leaf_any);
         }
 #endif
         if (inside) {
             p.dL_dray_o[3 * r + 0] = g_ro.x; p.dL_dray_o[3 * r + 1] = g_ro.y; p.dL_dray_o[3 * r + 2] = g_ro.z;
             p.dL_dray_d[3 * r + 0] = g_rd.x; p.dL_dray_d[3 * r + 1] = g_rd.y; p.dL_dray_d[3 * r + 2] = g_rd.z;
         }
-        // flush the block's table: consecutive threads take consecutive columns of a row, so the 48 SH
-        // columns of a surfel go out as contiguous atomics
         __syncthreads();
-        constexpr int stride = RowLayout<AUXM>::stride;
-        for (int k = threadIdx.x; k < kTableRows * stride; k += kWavesPerBlock * DST_WAVE) {
-            const int row = k / stride, col = k - row * stride;
-            const uint32_t g = s_keys[row];
-            if (g == kEmptyKey || col >= RowLayout<AUXM>::cols) continue;
-            const float v = s_rows[k];
-            if (v == 0.f) continue;
-            float *dst = grad_address<AUXM>(p, g, col);
-            if (dst != nullptr) aadd(dst, v);
-        }
+        table_flush<AUXM>(p, s_keys, s_rows);
     }
 }
 
