@@ -134,8 +134,8 @@ def main():
     A_total = A_fwd + A_bwd + PER_SURFEL_INIT * P
     rays_per_s = R / (ms_per_step * 1e-3)
 
-    dominant = ("backward", "k_trace_bwd<2,true>", A_bwd, bwd_ms) if bwd_ms >= fwd_ms else \
-        ("forward", "k_trace_fwd<2,true>", A_fwd, fwd_ms)
+    dominant = ("backward", "k_trace_bwd<2,true,false>", A_bwd, bwd_ms) if bwd_ms >= fwd_ms else \
+        ("forward", "k_trace_fwd<2,true,false>", A_fwd, fwd_ms)
     achieved = dominant[2] / (dominant[3] * 1e-3) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")

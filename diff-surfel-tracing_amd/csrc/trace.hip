@@ -354,8 +354,123 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
     }
 }
 
+// ---- per-lane walk ------------------------------------------------------------------------------------------
+// For rays that share neither origin nor direction (reflection rays off rough geometry, arbitrary ray lists) a
+// packet visits the union of 64 unrelated paths with one useful lane each.  Here every lane walks the hierarchy
+// on its own: own stack (private memory), own node and quad fetches through the vector path, same slab and
+// quad tests, same buffer.  The buffer's content does not depend on the order of arrival, so both walks give
+// the same result bit for bit; the choice between them only changes the time.
+#ifndef DST_PACKET_DIR_SPREAD
+#define DST_PACKET_DIR_SPREAD 0.06f
+#endif
+#ifndef DST_PACKET_ORG_SPREAD
+#define DST_PACKET_ORG_SPREAD 0.02f
+#endif
+constexpr float kPacketDirSpread = DST_PACKET_DIR_SPREAD;   // largest direction difference (relative) inside a packet
+constexpr float kPacketOrgSpread = DST_PACKET_ORG_SPREAD;   // largest origin difference, relative to the scene extent
+constexpr int kLaneStack = 3 * 64;        // as deep as the packet's three lane-indexed registers
+constexpr uint32_t kWalkDone = 0xFFFFFFFFu;   // not a reference: leaf bit set with an impossible position
+// A real call on purpose: inlined, its register needs would spill the packet walk that nearly every wave takes.
+__device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, const RaySlab &slab, F3 o, F3 d,
+                                                    bool active, KBuf &buf, uint32_t &cnt) {
+    RaySlabFast fs;
+    fs.ix = slab.ix; fs.iy = slab.iy; fs.iz = slab.iz;
+    fs.cnx = slab.nx - slab.wx; fs.cny = slab.ny - slab.wy; fs.cnz = slab.nz - slab.wz;
+    fs.cfx = slab.nx + slab.wx; fs.cfy = slab.ny + slab.wy; fs.cfz = slab.nz + slab.wz;
+    // float index of this lane's near / far face arrays inside a wide node (lox 0, loy 4, loz 8, hix 12, hiy 16, hiz 20)
+    const uint32_t onx = slab.ix < 0.f ? 12u : 0u, ofx = 12u - onx;
+    const uint32_t ony = slab.iy < 0.f ? 16u : 4u, ofy = 20u - ony;
+    const uint32_t onz = slab.iz < 0.f ? 20u : 8u, ofz = 28u - onz;
+    uint32_t stack[kLaneStack];
+    int sp = 0;
+    uint32_t ref = active ? acc.root : kWalkDone;
+    uint32_t budget = 2u * acc.n_leaves + 8u;   // a well-formed hierarchy needs fewer steps; bounds the loop regardless
+#pragma unroll 1
+    while (wave_ballot(ref != kWalkDone) != 0ull) {
+        if (ref == kWalkDone) continue;
+        uint32_t next = kWalkDone;
+        bool have_next = false;
+        if (ref & DST_LEAF_BIT) {
+            const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
+#pragma unroll 1
+            for (uint32_t q = 0; q < count && first + q < acc.n_leaves; ++q) {
+                const float *L = reinterpret_cast<const float *>(&acc.leaves[first + q]);
+                float t = 0.f;
+                uint32_t tri = 0u;
+                const bool hit = ray_quad(o, d, ld3(L), ld3(L + 3), ld3(L + 6), ld3(L + 9), ld3(L + 12), ld3(L + 15), t, tri);
+                const uint64_t x = kb_pack(t, 2u * __float_as_uint(L[18]) + tri);
+                const bool adm = hit && (x < buf.e[kChunk - 1]);
+                if (adm) {
+                    cnt += 1u;
+                    kbuf_insert(buf, x, true);
+                }
+            }
+        } else if (ref + 1u < acc.n_leaves) {
+            const float *N = reinterpret_cast<const float *>(&acc.wide[ref]);
+            const uint32_t *refs = reinterpret_cast<const uint32_t *>(N) + 24;
+            const uint32_t n_child = refs[4];
+            const float tmax = kb_t(buf.e[kChunk - 1]);
+            uint32_t key[DST_WIDE], cref[DST_WIDE];
+#pragma unroll
+            for (int k = 0; k < DST_WIDE; ++k) {
+                float tn;
+                const uint64_t h = slab_hit_fast(fs, N[onx + k], N[ony + k], N[onz + k], N[ofx + k], N[ofy + k],
+                                                 N[ofz + k], tmax, tn);
+                const bool mine = ((h >> __lane_id()) & 1ull) != 0ull && (uint32_t)k < n_child;
+                key[k] = mine ? __float_as_uint(tn) : 0xFFFFFFFFu;   // entry distance (non-negative: bits order like the value)
+                cref[k] = refs[k];
+            }
+#define CSWAP(a, b)                                                            \
+    {                                                                          \
+        const bool sw_ = key[b] < key[a];                                      \
+        const uint32_t ka_ = sw_ ? key[b] : key[a], kb_ = sw_ ? key[a] : key[b]; \
+        const uint32_t ra_ = sw_ ? cref[b] : cref[a], rb_ = sw_ ? cref[a] : cref[b]; \
+        key[a] = ka_; key[b] = kb_; cref[a] = ra_; cref[b] = rb_;              \
+    }
+            CSWAP(0, 1) CSWAP(2, 3) CSWAP(0, 2) CSWAP(1, 3) CSWAP(1, 2)
+#undef CSWAP
+            // defer the farther children (farthest first), go on with the nearest
+#pragma unroll
+            for (int k = DST_WIDE - 1; k >= 1; --k) {
+                if (key[k] != 0xFFFFFFFFu && sp < kLaneStack) stack[sp++] = cref[k];
+            }
+            if (key[0] != 0xFFFFFFFFu) {
+                next = cref[0];
+                have_next = true;
+            }
+        }
+        if (!have_next && sp > 0) {
+            next = stack[--sp];
+        }
+        ref = (--budget == 0u) ? kWalkDone : next;
+    }
+}
+
+// Packet or per-lane walk for the rays of this wave?  A packet pays off when the rays run side by side: every
+// live ray is compared with the first live one (origins as given by the caller, not advanced along the ray).
+__device__ __forceinline__ bool rays_run_together(F3 o, F3 d, bool active, float max_abs) {
+    const uint64_t live = wave_ballot(active);
+    if (live == 0ull) return true;
+    const int lead = __builtin_ctzll(live);
+    const F3 o0 = f3(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(o.x), lead)),
+                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(o.y), lead)),
+                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(o.z), lead)));
+    const F3 d0 = f3(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(d.x), lead)),
+                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d.y), lead)),
+                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d.z), lead)));
+    const float dd = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(d.x - d0.x), __builtin_fabsf(d.y - d0.y)),
+                                     __builtin_fabsf(d.z - d0.z));
+    const float od = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(o.x - o0.x), __builtin_fabsf(o.y - o0.y)),
+                                     __builtin_fabsf(o.z - o0.z));
+    const float dl = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(d0.x), __builtin_fabsf(d0.y)),
+                                     __builtin_fabsf(d0.z));
+    const bool apart = active && (!(dd <= kPacketDirSpread * dl) || !(od <= kPacketOrgSpread * max_abs));
+    return wave_ballot(apart) == 0ull;
+}
+
+template <bool MIXED>
 __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
-                                           uint32_t &cnt
+                                           uint32_t &cnt, bool as_packet
 #ifdef DST_STATS
                                            , WaveStats &ws
 #endif
@@ -363,6 +478,14 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
     const uint64_t live = wave_ballot(active);
     if (live == 0ull) return;
     const RaySlab slab = make_slab(o, d, max_abs);
+    if (MIXED && !as_packet) {
+        KBuf mine = buf;   // a copy the call may keep in memory; the caller's buffer stays in registers
+        uint32_t n = cnt;
+        lane_walk(acc, slab, o, d, active, mine, n);
+        buf = mine;
+        cnt = n;
+        return;
+    }
     // The walk assumes one set of direction signs per packet (the near face of every box is then the same for
     // all lanes).  A wave whose rays straddle an axis plane (about 1 % of the tiles of a pinhole image) is
     // walked once per sign class present, each time with the lanes of that class only.
@@ -827,7 +950,7 @@ __device__ __forceinline__ void table_clear_keys(uint32_t *keys) {
 
 // One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
 // and for BWD the per-hit gradients of the re-trace (reference backward.cu:332-655).
-template <bool BWD, int AUXM, bool REC>
+template <bool BWD, int AUXM, bool REC, bool MIXED>
 __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
@@ -847,6 +970,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     F3 ot = ro;
     bool live = lane_on;
     KBuf buf;
+    // kernels built without the per-lane walk (MIXED false) take every wave as a packet
+    const bool as_packet = (!MIXED || (REC && BWD)) ? true : rays_run_together(ro, rd, lane_on, max_abs);
     uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
     for (;;) {
         // Backward: the four waves of the block take their chunks in step, so that between two rounds nobody
@@ -869,7 +994,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             if (rec_block == nullptr) { live = false; break; }   // cannot happen with a complete record
         } else {
             kbuf_reset(buf);
-            packet_knn(acc, max_abs, ot, rd, live, buf, cnt WSP);
+            packet_knn<MIXED>(acc, max_abs, ot, rd, live, buf, cnt, as_packet WSP);
             if (REC && !BWD) rec_store(rv, bounce, rec_pos, buf, cnt);
         }
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
@@ -1035,7 +1160,7 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
     return v;
 }
 
-template <bool BWD, int AUXM, bool REC>
+template <bool BWD, int AUXM, bool REC, bool MIXED>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
@@ -1105,7 +1230,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i WS_ARG);
+            walk_bounce<false, AUXM, REC, MIXED>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -1245,7 +1370,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM, REC>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
+            walk_bounce<true, AUXM, REC, MIXED>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
         }
 #ifdef DST_STATS   // development build only: counters must then hold 11 entries
         if (p.counters != nullptr && lane == 0) {
@@ -1277,17 +1402,17 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
 #ifndef DST_BWD_WAVES
 #define DST_BWD_WAVES 3
 #endif
-template <int AUXM, bool REC>
+template <int AUXM, bool REC, bool MIXED>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x) {
-    trace_body<false, AUXM, REC>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+    trace_body<false, AUXM, REC, MIXED>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
 }
-template <int AUXM, bool REC>
+template <int AUXM, bool REC, bool MIXED>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
 void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x) {
-    trace_body<true, AUXM, REC>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+    trace_body<true, AUXM, REC, MIXED>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
 }
 
 struct TileGrid {
@@ -1315,18 +1440,27 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipS
         grid = dim3((t.btiles_x * t.btiles_y + 7u) / 8u * 32u);
         block = dim3(DST_WAVE);
     }
-#define DST_LAUNCH(AUX)                                                                                            \
+    // The per-lane walk is built into the kernels used where waves of unrelated rays are to be expected:
+    // reflection bounces and ray lists (thin grids).  Image-shaped grids traced to depth 0 get the pure packet kernels.
+    const bool mixed = p.max_trace_depth > 0 || t.th_log2 < 3;
+#define DST_LAUNCH_M(AUX, MIXED)                                                                                   \
     do {                                                                                                           \
         if (BWD)                                                                                                   \
-            hipLaunchKernelGGL((k_trace_bwd<AUX, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2,      \
-                               t.tiles_x, t.tiles_y, t.btiles_x);                                                  \
+            hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC>), grid, block, 0, stream, p, acc, t.tw_log2, \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                                       \
         else                                                                                                       \
-            hipLaunchKernelGGL((k_trace_fwd<AUX, REC>), grid, block, 0, stream, p, acc, t.tw_log2, t.th_log2,      \
-                               t.tiles_x, t.tiles_y, t.btiles_x);                                                  \
+            hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED>), grid, block, 0, stream, p, acc, t.tw_log2,          \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                                       \
+    } while (0)
+#define DST_LAUNCH(AUX)                                                                                            \
+    do {                                                                                                           \
+        if (mixed) DST_LAUNCH_M(AUX, true);                                                                        \
+        else DST_LAUNCH_M(AUX, false);                                                                             \
     } while (0)
     if (p.aux <= 2) DST_LAUNCH(2);
     else if (p.aux <= 4) DST_LAUNCH(4);
     else DST_LAUNCH(8);
+#undef DST_LAUNCH_M
 #undef DST_LAUNCH
 }
 
