@@ -89,6 +89,21 @@ def test_thin_ray_lists(oracle, tracer):
     check_case(oracle, tracer, sc, o3, d3, grads=False)
 
 
+def test_unrelated_rays_as_image_and_as_list(oracle, tracer):
+    """Random origins and directions (nothing for a packet to share): as an image-shaped grid the packet kernels
+    walk one direction-sign class at a time, as a ray list the per-lane walk takes over; both must equal the oracle
+    bit for bit, and hence each other."""
+    sc = S.scene_cube(P=6000, seed=77)
+    gen = torch.Generator().manual_seed(78)
+    n = 24 * 40
+    o = (torch.rand(n, 3, generator=gen) * 2 - 1) * 1.5
+    d = torch.nn.functional.normalize(torch.randn(n, 3, generator=gen), dim=-1)
+    _, a = check_case(oracle, tracer, sc, o.reshape(24, 40, 3).contiguous(), d.reshape(24, 40, 3).contiguous())
+    _, b = check_case(oracle, tracer, sc, o.reshape(1, n, 3).contiguous(), d.reshape(1, n, 3).contiguous())
+    for k in ("rgb", "dpt", "acc", "norm"):
+        assert np.array_equal(a[k].reshape(n, -1).view(np.uint32), b[k].reshape(n, -1).view(np.uint32)), k
+
+
 def test_ragged_image_sizes(oracle, tracer):
     sc = S.scene_cube(P=2000, seed=5)
     for H, W in ((37, 53), (1, 1), (9, 7), (64, 1)):
