@@ -168,25 +168,37 @@ __global__ void k_radix_hist(const uint32_t *__restrict__ keys, uint32_t *__rest
 
 // Exclusive scan of `len` counters in place, one block.
 __global__ void k_scan_exclusive(uint32_t *data, uint32_t len) {
-    __shared__ uint32_t part[1024];
-    const uint32_t t = threadIdx.x, nt = blockDim.x;
-    const uint32_t per = (len + nt - 1) / nt;
-    const uint32_t b = t * per, e = min(b + per, len);
-    uint32_t s = 0;
-    for (uint32_t i = b; i < e; ++i) s += data[i];
-    part[t] = s;
+    // one block walks the array in coalesced slabs of blockDim.x * 4 entries and carries the running total
+    __shared__ uint32_t wave_sum[1024 / DST_WAVE];
+    __shared__ uint32_t carry_s;
+    const uint32_t t = threadIdx.x, nt = blockDim.x, lane = t % DST_WAVE, w = t / DST_WAVE, nw = nt / DST_WAVE;
+    if (t == 0) carry_s = 0u;
     __syncthreads();
-    for (uint32_t off = 1; off < nt; off <<= 1) {
-        uint32_t v = (t >= off) ? part[t - off] : 0;
+    for (uint32_t base = 0; base < len; base += nt * 4u) {
+        const uint32_t i = base + t * 4u;
+        uint32_t v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = (i + k < len) ? data[i + k] : 0u;
+        const uint32_t mine = v[0] + v[1] + v[2] + v[3];
+        uint32_t incl = mine;   // inclusive scan over the wave
+#pragma unroll
+        for (int off = 1; off < DST_WAVE; off <<= 1) {
+            const uint32_t up = __shfl_up(incl, off);
+            if ((int)lane >= off) incl += up;
+        }
+        if (lane == DST_WAVE - 1) wave_sum[w] = incl;
         __syncthreads();
-        part[t] += v;
+        uint32_t before = carry_s;
+        for (uint32_t k = 0; k < w; ++k) before += wave_sum[k];
+        uint32_t run = before + incl - mine;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (i + k < len) data[i + k] = run;
+            run += v[k];
+        }
         __syncthreads();
-    }
-    uint32_t run = part[t] - s;
-    for (uint32_t i = b; i < e; ++i) {
-        uint32_t v = data[i];
-        data[i] = run;
-        run += v;
+        if (t == nt - 1) carry_s = run;   // the last thread's running total is the slab's
+        __syncthreads();
     }
 }
 
@@ -323,11 +335,20 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
     for (int k = 0; k < 5; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
 }
 
-// Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes.
+// Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes and goes on.
+// A node's leaves are contiguous and its index is the first or the last of them, so every node whose leaves
+// all belong to this block of kBlock consecutive leaves is reached only by threads of this block: those meet in
+// LDS (workgroup-scope ordering, no cache maintenance).  Only the few nodes that span blocks use the
+// agent-scope protocol through memory, whose fences write back and invalidate the L2 of the XCD.
 __global__ void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
                       const uint32_t *__restrict__ leaf_parent, uint32_t *flags, const DstLeaf *__restrict__ leaves,
                       uint32_t n) {
-    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ float s_box[kBlock][12];      // per local node: box of child 0, box of child 1
+    __shared__ uint32_t s_arrived[kBlock];
+    s_arrived[threadIdx.x] = 0u;
+    __syncthreads();
+    const uint32_t blk_lo = blockIdx.x * blockDim.x, blk_hi = min(blk_lo + blockDim.x, n) - 1u;
+    uint32_t i = blk_lo + threadIdx.x;
     if (i >= n) return;
     const DstLeaf &L = leaves[i];
     float box[6];
@@ -337,22 +358,42 @@ __global__ void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
         box[3 + a] = fmaxf(fmaxf(L.A[a], L.B[a]), fmaxf(L.C[a], L.D[a]));
     }
     uint32_t pp = leaf_parent[i];
+    bool local = true;
     while (pp != DST_NO_PARENT) {
         const uint32_t p = pp >> 1, which = pp & 1u;
         float *mine = which ? nodes[p].lo1 : nodes[p].lo0;
-        const float *other = which ? nodes[p].lo0 : nodes[p].lo1;
+        if (local) local = nodes[p].first >= blk_lo && nodes[p].last <= blk_hi;
+        if (local) {
+            const uint32_t slot = p - blk_lo;
 #pragma unroll
-        for (int k = 0; k < 6; ++k) __hip_atomic_store(mine + k, box[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        uint32_t arrived = atomicAdd(&flags[p], 1u);
-        if (arrived == 0) return;
-        __threadfence();
+            for (int k = 0; k < 6; ++k) {
+                mine[k] = box[k];                      // for the kernels that follow
+                s_box[slot][6 * which + k] = box[k];   // for the sibling's thread
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // the LDS stores come before the arrival count
+            const uint32_t arrived = __hip_atomic_fetch_add(&s_arrived[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (arrived == 0) return;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #pragma unroll
-        for (int k = 0; k < 3; ++k) {
-            float olo = __hip_atomic_load(other + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            float ohi = __hip_atomic_load(other + 3 + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            box[k] = fminf(box[k], olo);
-            box[3 + k] = fmaxf(box[3 + k], ohi);
+            for (int k = 0; k < 3; ++k) {
+                box[k] = fminf(box[k], s_box[slot][6 * (1u - which) + k]);
+                box[3 + k] = fmaxf(box[3 + k], s_box[slot][6 * (1u - which) + 3 + k]);
+            }
+        } else {
+            const float *other = which ? nodes[p].lo0 : nodes[p].lo1;
+#pragma unroll
+            for (int k = 0; k < 6; ++k) __hip_atomic_store(mine + k, box[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __threadfence();
+            uint32_t arrived = atomicAdd(&flags[p], 1u);
+            if (arrived == 0) return;
+            __threadfence();
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+                float olo = __hip_atomic_load(other + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                float ohi = __hip_atomic_load(other + 3 + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                box[k] = fminf(box[k], olo);
+                box[3 + k] = fmaxf(box[3 + k], ohi);
+            }
         }
         pp = node_parent[p];
     }
