@@ -58,11 +58,12 @@ template <bool REBUILD>
 __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vertices,
                              const int32_t *__restrict__ triangles, int4 *__restrict__ quad_ids,
                              float4 *__restrict__ centroids, DstBounds *__restrict__ bounds, uint32_t P) {
-    uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
-    float lo[3] = {INFINITY, INFINITY, INFINITY}, hi[3] = {-INFINITY, -INFINITY, -INFINITY};
+    // grid-stride: a wave ends with seven atomics on the same seven words, and those are served one by one,
+    // so each wave takes many surfels
     float cen[3] = {INFINITY, INFINITY, INFINITY}, cenh[3] = {-INFINITY, -INFINITY, -INFINITY};
     float mabs = 0.f;
-    if (g < P) {
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < P; g += gridDim.x * blockDim.x) {
+        float lo[3] = {INFINITY, INFINITY, INFINITY}, hi[3] = {-INFINITY, -INFINITY, -INFINITY};
         int4 q;
         if (REBUILD) {
             const int32_t *t = triangles + (size_t)g * 6;
@@ -96,9 +97,9 @@ __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vert
         c4.z = 0.5f * (lo[2] + hi[2]);
         c4.w = 0.f;
         centroids[g] = c4;
-        cen[0] = cenh[0] = c4.x;
-        cen[1] = cenh[1] = c4.y;
-        cen[2] = cenh[2] = c4.z;
+        cen[0] = fminf(cen[0], c4.x); cenh[0] = fmaxf(cenh[0], c4.x);
+        cen[1] = fminf(cen[1], c4.y); cenh[1] = fmaxf(cenh[1], c4.y);
+        cen[2] = fminf(cen[2], c4.z); cenh[2] = fmaxf(cenh[2], c4.z);
     }
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -171,15 +172,18 @@ __global__ void k_scan_exclusive(uint32_t *data, uint32_t len) {
     // one block walks the array in coalesced slabs of blockDim.x * 4 entries and carries the running total
     __shared__ uint32_t wave_sum[1024 / DST_WAVE];
     __shared__ uint32_t carry_s;
+    constexpr uint32_t kPer = 4u;
     const uint32_t t = threadIdx.x, nt = blockDim.x, lane = t % DST_WAVE, w = t / DST_WAVE, nw = nt / DST_WAVE;
     if (t == 0) carry_s = 0u;
     __syncthreads();
-    for (uint32_t base = 0; base < len; base += nt * 4u) {
-        const uint32_t i = base + t * 4u;
-        uint32_t v[4];
+    for (uint32_t base = 0; base < len; base += nt * kPer) {
+        const uint32_t i = base + t * kPer;
+        uint32_t v[kPer];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] = (i + k < len) ? data[i + k] : 0u;
-        const uint32_t mine = v[0] + v[1] + v[2] + v[3];
+        for (int k = 0; k < (int)kPer; ++k) v[k] = (i + k < len) ? data[i + k] : 0u;
+        uint32_t mine = 0u;
+#pragma unroll
+        for (int k = 0; k < (int)kPer; ++k) mine += v[k];
         uint32_t incl = mine;   // inclusive scan over the wave
 #pragma unroll
         for (int off = 1; off < DST_WAVE; off <<= 1) {
@@ -192,7 +196,7 @@ __global__ void k_scan_exclusive(uint32_t *data, uint32_t len) {
         for (uint32_t k = 0; k < w; ++k) before += wave_sum[k];
         uint32_t run = before + incl - mine;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < (int)kPer; ++k) {
             if (i + k < len) data[i + k] = run;
             run += v[k];
         }
@@ -337,14 +341,15 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
 
 // Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes and goes on.
 // A node's leaves are contiguous and its index is the first or the last of them, so every node whose leaves
-// all belong to this block of kBlock consecutive leaves is reached only by threads of this block: those meet in
+// all belong to this block of kFitBlock consecutive leaves is reached only by threads of this block: those meet in
 // LDS (workgroup-scope ordering, no cache maintenance).  Only the few nodes that span blocks use the
 // agent-scope protocol through memory, whose fences write back and invalidate the L2 of the XCD.
-__global__ void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
+constexpr int kFitBlock = 1024;
+__global__ __launch_bounds__(kFitBlock) void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
                       const uint32_t *__restrict__ leaf_parent, uint32_t *flags, const DstLeaf *__restrict__ leaves,
                       uint32_t n) {
-    __shared__ float s_box[kBlock][12];      // per local node: box of child 0, box of child 1
-    __shared__ uint32_t s_arrived[kBlock];
+    __shared__ float s_box[kFitBlock][12];      // per local node: box of child 0, box of child 1
+    __shared__ uint32_t s_arrived[kFitBlock];
     s_arrived[threadIdx.x] = 0u;
     __syncthreads();
     const uint32_t blk_lo = blockIdx.x * blockDim.x, blk_hi = min(blk_lo + blockDim.x, n) - 1u;
@@ -511,11 +516,12 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     float4 *centroids = reinterpret_cast<float4 *>(ctx->centroids);
 
     hipLaunchKernelGGL(k_init_bounds, dim3(1), dim3(64), 0, stream, ctx->bounds);
+    const dim3 setup_grid(std::min<uint32_t>(grid_for(n).x, 1024u));   // 4 blocks per CU, each thread takes several surfels
     if (rebuild)
-        hipLaunchKernelGGL(k_quad_setup<true>, grid_for(n), dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
+        hipLaunchKernelGGL(k_quad_setup<true>, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
                            quad_ids, centroids, ctx->bounds, n);
     else
-        hipLaunchKernelGGL(k_quad_setup<false>, grid_for(n), dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
+        hipLaunchKernelGGL(k_quad_setup<false>, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
                            quad_ids, centroids, ctx->bounds, n);
 
     if (rebuild) {
@@ -544,7 +550,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0], ctx->leaves,
                        n);
     hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->flags, 0u, n);
-    hipLaunchKernelGGL(k_fit, grid_for(n), dim3(kBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
+    hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
                        ctx->flags, ctx->leaves, n);
     if (n > DST_GROUP)
         hipLaunchKernelGGL(k_widen, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, ctx->wide, n - 1);
