@@ -1000,14 +1000,35 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
         int here = 0;
         bool stop = false;
+        // Replay runs one step ahead of itself: the entry of step it+1 is fetched while step it evaluates, and its
+        // surfel's geometry while step it does its gradient algebra, so a step starts with its operands in registers
+        // instead of two dependent trips to memory.
+        struct Ahead { uint64_t e; float m[3], s[2], q[4], o; } nx = {0ull, {0.f, 0.f, 0.f}, {1.f, 1.f}, {1.f, 0.f, 0.f, 0.f}, 0.f};
+        auto fetch_geometry = [&](bool want) {
+            if (!want) return;
+            const size_t gn = (size_t)(kb_idx(nx.e) >> 1);
+            nx.m[0] = p.means3D[3 * gn]; nx.m[1] = p.means3D[3 * gn + 1]; nx.m[2] = p.means3D[3 * gn + 2];
+            nx.s[0] = p.scales[2 * gn]; nx.s[1] = p.scales[2 * gn + 1];
+            nx.q[0] = p.rotations[4 * gn]; nx.q[1] = p.rotations[4 * gn + 1];
+            nx.q[2] = p.rotations[4 * gn + 2]; nx.q[3] = p.rotations[4 * gn + 3];
+            nx.o = p.opacities[gn];
+        };
+        if (REC && BWD) {
+            const bool want = live && cnt > 0u;
+            if (want) nx.e = rec_block[lane_];
+            fetch_geometry(want);
+        }
 #pragma unroll 1
         for (int it = 0; it < kChunk; ++it) {
             const bool on = live && !stop && (uint32_t)it < cnt;
             if (wave_ballot(on) == 0ull) break;
             // next entry in depth order (consumed slots need no reset: the buffer is rebuilt for every chunk)
             uint64_t e;
+            Ahead cur = nx;
+            const bool want_next = (REC && BWD) && live && it + 1 < kChunk && (uint32_t)(it + 1) < cnt;
             if (REC && BWD) {
-                e = rec_block[it * DST_WAVE + lane_];
+                e = cur.e;
+                if (want_next) nx.e = rec_block[(it + 1) * DST_WAVE + lane_];
             } else {
                 e = buf.e[0];
 #pragma unroll
@@ -1031,11 +1052,17 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 if (g == last_g) break;
                 dpt = e_t + pay_dpt;
                 xyz = f3(ro.x + dpt * rd.x, ro.y + dpt * rd.y, ro.z + dpt * rd.z);
-                mean = ld3(p.means3D + 3 * (size_t)g);
-                sx = p.scales[2 * (size_t)g];
-                sy = p.scales[2 * (size_t)g + 1];
-                const float *qp = p.rotations + 4 * (size_t)g;
-                q0 = qp[0]; q1 = qp[1]; q2 = qp[2]; q3 = qp[3];
+                if (REC && BWD) {
+                    mean = f3(cur.m[0], cur.m[1], cur.m[2]);
+                    sx = cur.s[0]; sy = cur.s[1];
+                    q0 = cur.q[0]; q1 = cur.q[1]; q2 = cur.q[2]; q3 = cur.q[3];
+                } else {
+                    mean = ld3(p.means3D + 3 * (size_t)g);
+                    sx = p.scales[2 * (size_t)g];
+                    sy = p.scales[2 * (size_t)g + 1];
+                    const float *qp = p.rotations + 4 * (size_t)g;
+                    q0 = qp[0]; q1 = qp[1]; q2 = qp[2]; q3 = qp[3];
+                }
                 quat_rows(q0, q1, q2, q3, R);
                 const float Tx = dot(R[0], mean), Ty = dot(R[1], mean);
                 const float ux = R[0].x * xyz.x + R[0].y * xyz.y + R[0].z * xyz.z + (-Tx);
@@ -1052,7 +1079,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 if (dpt < min_depth) break;
                 const float power = -0.5f * rho;
                 if (power > 0.0f) break;
-                opac = p.opacities[g];
+                opac = (REC && BWD) ? cur.o : p.opacities[g];
                 G = exp_det(power);
                 alpha = opac * G;
                 alpha = (alpha < 0.99f) ? alpha : 0.99f;
@@ -1091,6 +1118,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 dpt_hit = dpt;
                 Tp = Tn;
             } while (false);
+            if (REC && BWD) fetch_geometry(want_next);
             if (!BWD && p.training && p.a_weights != nullptr) wave_add_grouped(p.a_weights, did, (uint32_t)g, w);
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
             if (BWD && wave_ballot(did) != 0ull) {
