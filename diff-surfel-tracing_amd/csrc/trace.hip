@@ -300,10 +300,10 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
             const char *node = reinterpret_cast<const char *>(&acc.wide[ref]);
             STAT(ws.nodes++;)
             const float tmax = active ? kb_t(buf.e[kChunk - 1]) : -1.0f;
-            uint32_t key[DST_WIDE], cref[DST_WIDE], tail[5];
+            uint32_t tail[5];
             load_uniform<5>(node + 96, tail);      // ref[4], count
             const uint32_t n_child = tail[4];
-            int n_push = 0;
+            uint32_t hit = 0u;                     // bit k: some lane enters child k
             {
                 uint32_t NX[4], NY[4], NZ[4], FX[4], FY[4], FZ[4];
                 load_uniform<4>(node + onx, NX); load_uniform<4>(node + ony, NY); load_uniform<4>(node + onz, NZ);
@@ -314,37 +314,27 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                     const uint64_t h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
                                                      __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
                                                      __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn);
-                    // Key: entry distance of the representative lane if it hits the child itself (non-negative,
-                    // so its bits order like the value), +inf if only other lanes do, all ones if nobody does or
-                    // the slot is unused.
-                    const uint32_t kk = __builtin_amdgcn_readlane(__float_as_uint(tn), rep);
-                    const uint32_t mine = ((h >> rep) & 1ull) ? kk : 0x7F800000u;
-                    key[k] = ((uint32_t)k < n_child && h != 0ull) ? mine : 0xFFFFFFFFu;
-                    cref[k] = tail[k];
+                    hit |= (h != 0ull) ? (1u << k) : 0u;
                 }
-                n_push = 4 - (int)((key[0] >> 31) + (key[1] >> 31) + (key[2] >> 31) + (key[3] >> 31));
+                hit &= (1u << n_child) - 1u;       // unused slots are never entered
             }
-            if (n_push > 0) {
-                // sort the four (key, ref) pairs, nearest first; children nobody wants carry the largest key
-#define CSWAP(a, b)                                                            \
-    {                                                                          \
-        const bool sw_ = key[b] < key[a];                                      \
-        const uint32_t ka_ = sw_ ? key[b] : key[a], kb_ = sw_ ? key[a] : key[b]; \
-        const uint32_t ra_ = sw_ ? cref[b] : cref[a], rb_ = sw_ ? cref[a] : cref[b]; \
-        key[a] = ka_; key[b] = kb_; cref[a] = ra_; cref[b] = rb_;              \
+            if (hit != 0u) {
+                // Children are taken in stored order: the first one that is hit next, the others deferred (last
+                // first).  Ordering them by entry distance was measured: 3 % fewer visits, but the scalar work of
+                // the sort costs more than those visits.
+#define DST_PUSH(v)                                                     \
+    {                                                                   \
+        const uint32_t slot = (uint32_t)sp & 63u;                       \
+        if (sp < 64) stack0 = (lane == slot) ? (v) : stack0;            \
+        else if (sp < 128) stack1 = (lane == slot) ? (v) : stack1;      \
+        else stack2 = (lane == slot) ? (v) : stack2;                    \
+        ++sp;                                                           \
     }
-                CSWAP(0, 1) CSWAP(2, 3) CSWAP(0, 2) CSWAP(1, 3) CSWAP(1, 2)
-#undef CSWAP
-                // defer the farther ones (farthest first), continue with the nearest
-                for (int k = n_push - 1; k >= 1; --k) {
-                    const uint32_t v = cref[k];
-                    const uint32_t slot = (uint32_t)sp & 63u;
-                    if (sp < 64) stack0 = (lane == slot) ? v : stack0;
-                    else if (sp < 128) stack1 = (lane == slot) ? v : stack1;
-                    else stack2 = (lane == slot) ? v : stack2;
-                    ++sp;
-                }
-                ref = cref[0];
+                if ((hit & 8u) && (hit & 7u)) DST_PUSH(tail[3])
+                if ((hit & 4u) && (hit & 3u)) DST_PUSH(tail[2])
+                if ((hit & 2u) && (hit & 1u)) DST_PUSH(tail[1])
+#undef DST_PUSH
+                ref = (hit & 1u) ? tail[0] : ((hit & 2u) ? tail[1] : ((hit & 4u) ? tail[2] : tail[3]));
                 continue;
             }
         }
