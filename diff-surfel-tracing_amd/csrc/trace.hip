@@ -263,8 +263,8 @@ __device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool 
 
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
 // to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow: nodes and quads
-// are fetched once per wave, the stack is three VGPRs addressed by lane (192 entries: the binary hierarchy
-// is at most 62 levels deep and each 4-wide step defers at most three children).
+// are fetched once per wave, the stack is two VGPRs addressed by lane (128 entries: the binary hierarchy
+// is at most 62 levels deep, a 4-wide step goes down two of them and defers at most three children: 96).
 // All active lanes share the direction signs `sgn` (bit a set = axis a negative), see slab_hit_fast.
 __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySlab &slab, uint32_t sgn, F3 o, F3 d,
                                             bool active, int rep, KBuf &buf, uint32_t &cnt
@@ -285,7 +285,7 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
     if (sgn & 1u) { onx = 48; ofx = 0; }
     if (sgn & 2u) { ony = 64; ofy = 16; }
     if (sgn & 4u) { onz = 80; ofz = 32; }
-    uint32_t stack0 = 0u, stack1 = 0u, stack2 = 0u;
+    uint32_t stack0 = 0u, stack1 = 0u;
     int sp = 0;
     uint32_t ref = acc.root;
     // A well-formed hierarchy is walked in at most one step per node and per leaf group; the cap makes the
@@ -322,13 +322,13 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                 // Children are taken in stored order: the first one that is hit next, the others deferred (last
                 // first).  Ordering them by entry distance was measured: 3 % fewer visits, but the scalar work of
                 // the sort costs more than those visits.
-#define DST_PUSH(v)                                                     \
-    {                                                                   \
-        const uint32_t slot = (uint32_t)sp & 63u;                       \
-        if (sp < 64) stack0 = (lane == slot) ? (v) : stack0;            \
-        else if (sp < 128) stack1 = (lane == slot) ? (v) : stack1;      \
-        else stack2 = (lane == slot) ? (v) : stack2;                    \
-        ++sp;                                                           \
+#define DST_PUSH(v)                                                                   \
+    {   /* no lane has the number 255: the register that is not meant keeps its content */ \
+        const uint32_t slot = (uint32_t)sp & 63u;                                     \
+        const uint32_t t0 = sp < 64 ? slot : 255u, t1 = sp < 64 ? 255u : slot;        \
+        stack0 = (lane == t0) ? (v) : stack0;                                         \
+        stack1 = (lane == t1) ? (v) : stack1;                                         \
+        sp = min(sp + 1, 2 * DST_WAVE - 1);                                           \
     }
                 if ((hit & 8u) && (hit & 7u)) DST_PUSH(tail[3])
                 if ((hit & 4u) && (hit & 3u)) DST_PUSH(tail[2])
@@ -340,7 +340,10 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
         }
         if (sp == 0) break;
         --sp;
-        ref = __builtin_amdgcn_readlane(sp < 64 ? stack0 : (sp < 128 ? stack1 : stack2), sp & 63);
+        {
+            const uint32_t a = __builtin_amdgcn_readlane(stack0, sp & 63), b = __builtin_amdgcn_readlane(stack1, sp & 63);
+            ref = sp < 64 ? a : b;
+        }
     }
 }
 
@@ -358,7 +361,7 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
 #endif
 constexpr float kPacketDirSpread = DST_PACKET_DIR_SPREAD;   // largest direction difference (relative) inside a packet
 constexpr float kPacketOrgSpread = DST_PACKET_ORG_SPREAD;   // largest origin difference, relative to the scene extent
-constexpr int kLaneStack = 3 * 64;        // as deep as the packet's three lane-indexed registers
+constexpr int kLaneStack = 2 * 64;        // as deep as the packet's two lane-indexed registers
 constexpr uint32_t kWalkDone = 0xFFFFFFFFu;   // not a reference: leaf bit set with an impossible position
 // A real call on purpose: inlined, its register needs would spill the packet walk that nearly every wave takes.
 __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, const RaySlab &slab, F3 o, F3 d,
