@@ -9,6 +9,20 @@
  * Hit enumeration (owned by NVIDIA OptiX in the reference, which is not part
  * of the reference tree) is DEFINED here, see surfel_oracle.cpp: parity of
  * that part against OptiX itself is unpinned.
+ *
+ * Parity unpinned (transcribed from the cited lines and reviewed, but checked
+ * by no independent test, because the reference deviates from the true
+ * gradient there and nothing but the reference itself says how):
+ *   - bounce_backward(): the flow of dL/dacc (the reference never accumulates
+ *     the weight sum W, backward.cu:568);
+ *   - path_backward(): the part of a bounce's gradient that reaches the
+ *     previous bounce through the reflected ray's origin and direction
+ *     (backward.cu:700-790).
+ * Everything else is pinned by tests/test_oracle_*.py: scalar functions against
+ * numpy/scipy, the ray/quad test against float64 Moeller-Trumbore, hit ordering
+ * against brute force, compositing against closed forms, gradients (depth 0
+ * and the bounce weighting at depth 1) against torch autograd of an
+ * independent float64 forward.
  */
 #ifndef SURFEL_ORACLE_H
 #define SURFEL_ORACLE_H

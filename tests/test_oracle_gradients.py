@@ -224,3 +224,85 @@ def test_sh_mode_replaces_ray_direction_gradient(oracle):
     col = torch.clamp((sh_basis(d64)[:, None, :, None] * shs[None]).sum(2) + 0.5, min=0.0)[0, 0]
     (col * up["rgb"].double()[0] * w).sum().backward()
     np.testing.assert_allclose(got["ray_d"].ravel(), d64.grad.numpy().ravel(), rtol=1e-4, atol=1e-7)
+
+
+def test_second_bounce_gradients_match_autograd_with_the_reflected_rays_held_fixed(oracle):
+    """Pins how the bounces are combined in the backward pass (backward.cu:658-790: the weights f_i * prod s_j, the
+    per-bounce upstream gradients) and the compositing gradients of a bounce > 0.
+
+    Scene: a "mirror" cluster A around z = 0 facing a camera at z = 2, and a cluster B above the camera that only
+    the reflected rays can reach.  The float64 model renders bounce 0 from the camera rays and bounce 1 from the
+    reflected rays the oracle itself reports in mid_val, held fixed; out = C0 (1 - O0[0]) + C1 O0[0].  Holding the
+    reflected rays fixed removes exactly the part of the gradient that flows through the reflection geometry (and
+    that the reference approximates), so the comparison is made where that part is absent: every parameter of the
+    surfels that only bounce 1 hits, and the colours and aux channels of all surfels."""
+    gen = torch.Generator().manual_seed(11)
+    PA, PB, R = 40, 60, 48
+    meansA = torch.cat([(torch.rand(PA, 2, generator=gen) * 2 - 1) * 0.45, 0.02 * torch.randn(PA, 1, generator=gen)], -1)
+    qA = torch.tensor([1.0, 0.0, 0.0, 0.0]) + 0.08 * torch.randn(PA, 4, generator=gen)     # normals close to +z
+    meansB = torch.cat([(torch.rand(PB, 2, generator=gen) * 2 - 1) * 0.9, 3.2 + 0.3 * torch.rand(PB, 1, generator=gen)], -1)
+    qB = torch.randn(PB, 4, generator=gen)
+    means = torch.cat([meansA, meansB])
+    q = torch.cat([qA, qB])
+    q = q / q.norm(dim=-1, keepdim=True)
+    scales = torch.cat([torch.exp(-1.6 + 0.2 * torch.randn(PA, 2, generator=gen)),
+                        torch.exp(-1.3 + 0.3 * torch.randn(PB, 2, generator=gen))])
+    opac = torch.sigmoid(1.0 + torch.randn(PA + PB, 1, generator=gen))
+    others = torch.rand(PA + PB, 2, generator=gen)
+    others[:PA, 0] = 0.5 + 0.4 * others[:PA, 0]                                            # specular of the mirror
+    sc = {"means3D": means, "scales": scales, "rotations": q, "opacities": opac,
+          "colors_precomp": torch.rand(PA + PB, 3, generator=gen), "others_precomp": others}
+    sc = {k: v.float().contiguous() for k, v in sc.items()}
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    ro = torch.tensor([0.0, 0.0, 2.0]) + 0.03 * torch.randn(R, 3, generator=gen)
+    target = torch.cat([(torch.rand(R, 2, generator=gen) * 2 - 1) * 0.3, torch.zeros(R, 1)], -1)
+    rd = target - ro
+    rd = (rd / rd.norm(dim=-1, keepdim=True)).float().contiguous()
+    ro = ro.float().contiguous()
+    g_rgb = torch.randn(R, 3, generator=gen)
+
+    s = oracle_scene(oracle, sc, ro.reshape(1, R, 3), rd.reshape(1, R, 3), max_trace_depth=1, specular_threshold=0.1)
+    fwd = oracle.forward(s, oracle.HITS_BRUTE_LEXI)
+    got = oracle.backward(s, fwd, {"rgb": g_rgb.reshape(1, R, 3).numpy()}, oracle.HITS_BRUTE_LEXI)
+    MID = 14 + 2
+    mid = torch.from_numpy(fwd["mid"].reshape(R, 2, MID)).double()
+    o1, d1 = mid[:, 1, 0:3], mid[:, 1, 3:6]
+    bounced = d1.norm(dim=-1) > 0
+    assert bounced.sum() > R // 2, "the mirror must reflect most rays"
+
+    leaf = {k: sc[k].double().requires_grad_(True) for k in sc if k not in ("vertices", "faces")}
+    zero_bg = torch.zeros(3, dtype=torch.float64)
+    args = dict(colors=leaf["colors_precomp"], others=leaf["others_precomp"])
+    geo = (leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["opacities"], zero_bg)
+    C0, D0, N0, O0, info0 = forward64(ro.double(), rd.double(), *geo, **args)
+    d1_safe = torch.where(bounced[:, None], d1, torch.tensor([0.0, 0.0, 1.0], dtype=torch.float64).expand(R, 3))
+    C1, _, _, _, info1 = forward64(o1, d1_safe, *geo, near=0.06, **args)
+    C1 = torch.where(bounced[:, None], C1, torch.zeros_like(C1))
+    out = C0 * (1 - O0[:, :1]) + C1 * O0[:, :1]
+    # same function: bounce colours, the combined colour and the hit counts of both bounces agree
+    np.testing.assert_allclose(fwd["rgb"].reshape(R, 3), out.detach().numpy(), atol=3e-5)
+    np.testing.assert_allclose(mid[:, 0, 13:16].numpy(), C0.detach().numpy(), atol=3e-5)
+    np.testing.assert_allclose(mid[bounced][:, 1, 13:16].numpy(), C1[bounced].detach().numpy(), atol=3e-5)
+    n1 = torch.where(bounced, info1["n_con"], torch.zeros_like(info1["n_con"]))
+    np.testing.assert_array_equal(fwd["n_con"].reshape(R), (info0["n_con"] + n1).numpy())
+    assert n1.sum() > R, "bounce 1 must composite hits"
+
+    (out * g_rgb.double()).sum().backward()
+
+    def check(name, mine, want, rows, rel=2e-3):
+        mine, want = np.asarray(mine, np.float64).reshape(want.shape)[rows], want.numpy()[rows]
+        scale = np.abs(want).max()
+        assert scale > 0, name
+        err = np.abs(mine - want).max() / scale
+        assert err < rel, "%s: relative error %.3g" % (name, err)
+
+    B = slice(PA, PA + PB)   # never seen by the camera rays: z > 3 is behind their origin
+    check("means3D of B", got["means3D"], leaf["means3D"].grad, B)
+    check("scales of B", got["scales"], leaf["scales"].grad, B)
+    check("opacities of B", got["opacities"], leaf["opacities"].grad, B)
+    qn = sc["rotations"].double().numpy()
+    proj = got["rotations"].astype(np.float64) - qn * (qn * got["rotations"]).sum(-1, keepdims=True)
+    check("rotations of B", proj, leaf["rotations"].grad, B)
+    check("colours of all", got["colors_precomp"], leaf["colors_precomp"].grad, slice(0, PA + PB))
+    # the specular channel of the mirror weighs the two bounces against each other: d out / d O0 = C1 - C0
+    check("aux channels of all", got["others_precomp"], leaf["others_precomp"].grad, slice(0, PA + PB))
