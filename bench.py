@@ -52,7 +52,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (rays would be sharded across "
-              "GPUs with one all-reduce of the per-surfel gradients, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "GPUs with one all-reduce of the per-surfel gradients)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
