@@ -364,8 +364,11 @@ constexpr float kPacketOrgSpread = DST_PACKET_ORG_SPREAD;   // largest origin di
 constexpr int kLaneStack = 2 * 64;        // as deep as the packet's two lane-indexed registers
 constexpr uint32_t kWalkDone = 0xFFFFFFFFu;   // not a reference: leaf bit set with an impossible position
 // A real call on purpose: inlined, its register needs would spill the packet walk that nearly every wave takes.
+// `shelf`: optional LDS for the first kLaneShelf stack entries of every lane ([entry][lane], conflict-free);
+// deeper entries, or all of them without a shelf, live in private memory.
+constexpr int kLaneShelf = 32;
 __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, const RaySlab &slab, F3 o, F3 d,
-                                                    bool active, KBuf &buf, uint32_t &cnt) {
+                                                    bool active, KBuf &buf, uint32_t &cnt, uint32_t *shelf) {
     RaySlabFast fs;
     fs.ix = slab.ix; fs.iy = slab.iy; fs.iz = slab.iz;
     fs.cnx = slab.nx - slab.wx; fs.cny = slab.ny - slab.wy; fs.cnz = slab.nz - slab.wz;
@@ -425,7 +428,11 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
             // defer the farther children (farthest first), go on with the nearest
 #pragma unroll
             for (int k = DST_WIDE - 1; k >= 1; --k) {
-                if (key[k] != 0xFFFFFFFFu && sp < kLaneStack) stack[sp++] = cref[k];
+                if (key[k] != 0xFFFFFFFFu && sp < kLaneStack) {
+                    if (shelf != nullptr && sp < kLaneShelf) shelf[sp * DST_WAVE + (int)__lane_id()] = cref[k];
+                    else stack[sp] = cref[k];
+                    ++sp;
+                }
             }
             if (key[0] != 0xFFFFFFFFu) {
                 next = cref[0];
@@ -433,7 +440,8 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
             }
         }
         if (!have_next && sp > 0) {
-            next = stack[--sp];
+            --sp;
+            next = (shelf != nullptr && sp < kLaneShelf) ? shelf[sp * DST_WAVE + (int)__lane_id()] : stack[sp];
         }
         ref = (--budget == 0u) ? kWalkDone : next;
     }
@@ -461,7 +469,7 @@ __device__ __forceinline__ bool rays_run_together(F3 o, F3 d, bool active, float
     return wave_ballot(apart) == 0ull;
 }
 
-template <bool MIXED>
+template <bool MIXED, bool SHELF>
 __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
                                            uint32_t &cnt, bool as_packet
 #ifdef DST_STATS
@@ -474,7 +482,10 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
     if (MIXED && !as_packet) {
         KBuf mine = buf;   // a copy the call may keep in memory; the caller's buffer stays in registers
         uint32_t n = cnt;
-        lane_walk(acc, slab, o, d, active, mine, n);
+        // forward kernels (one wave per workgroup, no other LDS) give the walk an LDS shelf for its stacks
+        __shared__ uint32_t s_shelf[SHELF ? kFwdWavesPerBlock * kLaneShelf * DST_WAVE : 1];
+        lane_walk(acc, slab, o, d, active, mine, n,
+                  SHELF ? s_shelf + (threadIdx.x / DST_WAVE) * (kLaneShelf * DST_WAVE) : nullptr);
         buf = mine;
         cnt = n;
         return;
@@ -987,7 +998,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             if (rec_block == nullptr) { live = false; break; }   // cannot happen with a complete record
         } else {
             kbuf_reset(buf);
-            packet_knn<MIXED>(acc, max_abs, ot, rd, live, buf, cnt, as_packet WSP);
+            packet_knn<MIXED, MIXED && !BWD>(acc, max_abs, ot, rd, live, buf, cnt, as_packet WSP);
             if (REC && !BWD) rec_store(rv, bounce, rec_pos, buf, cnt);
         }
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
