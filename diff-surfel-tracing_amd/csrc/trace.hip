@@ -364,6 +364,11 @@ constexpr float kPacketOrgSpread = DST_PACKET_ORG_SPREAD;   // largest origin di
 constexpr int kLaneStack = 2 * 64;        // as deep as the packet's two lane-indexed registers
 constexpr uint32_t kWalkDone = 0xFFFFFFFFu;   // not a reference: leaf bit set with an impossible position
 // A real call on purpose: inlined, its register needs would spill the packet walk that nearly every wave takes.
+// The walk is a real function, so the compiler cannot see where its pointers lead: say it (global memory, LDS).
+typedef const __attribute__((address_space(1))) float *global_f32;
+typedef const __attribute__((address_space(1))) uint32_t *global_u32;
+typedef __attribute__((address_space(3))) uint32_t *lds_u32;
+#define LD3(p, k) f3((p)[(k)], (p)[(k) + 1], (p)[(k) + 2])
 // `shelf`: optional LDS for the first kLaneShelf stack entries of every lane ([entry][lane], conflict-free);
 // deeper entries, or all of them without a shelf, live in private memory.
 constexpr int kLaneShelf = 32;
@@ -390,10 +395,10 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
             const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
 #pragma unroll 1
             for (uint32_t q = 0; q < count && first + q < acc.n_leaves; ++q) {
-                const float *L = reinterpret_cast<const float *>(&acc.leaves[first + q]);
+                const global_f32 L = (global_f32)reinterpret_cast<const float *>(&acc.leaves[first + q]);
                 float t = 0.f;
                 uint32_t tri = 0u;
-                const bool hit = ray_quad(o, d, ld3(L), ld3(L + 3), ld3(L + 6), ld3(L + 9), ld3(L + 12), ld3(L + 15), t, tri);
+                const bool hit = ray_quad(o, d, LD3(L, 0), LD3(L, 3), LD3(L, 6), LD3(L, 9), LD3(L, 12), LD3(L, 15), t, tri);
                 const uint64_t x = kb_pack(t, 2u * __float_as_uint(L[18]) + tri);
                 const bool adm = hit && (x < buf.e[kChunk - 1]);
                 if (adm) {
@@ -402,8 +407,8 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
                 }
             }
         } else if (ref + 1u < acc.n_leaves) {
-            const float *N = reinterpret_cast<const float *>(&acc.wide[ref]);
-            const uint32_t *refs = reinterpret_cast<const uint32_t *>(N) + 24;
+            const global_f32 N = (global_f32)reinterpret_cast<const float *>(&acc.wide[ref]);
+            const global_u32 refs = (global_u32)reinterpret_cast<const uint32_t *>(&acc.wide[ref]) + 24;
             const uint32_t n_child = refs[4];
             const float tmax = kb_t(buf.e[kChunk - 1]);
             uint32_t key[DST_WIDE], cref[DST_WIDE];
@@ -429,7 +434,7 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
 #pragma unroll
             for (int k = DST_WIDE - 1; k >= 1; --k) {
                 if (key[k] != 0xFFFFFFFFu && sp < kLaneStack) {
-                    if (shelf != nullptr && sp < kLaneShelf) shelf[sp * DST_WAVE + (int)__lane_id()] = cref[k];
+                    if (shelf != nullptr && sp < kLaneShelf) ((lds_u32)shelf)[sp * DST_WAVE + (int)__lane_id()] = cref[k];
                     else stack[sp] = cref[k];
                     ++sp;
                 }
@@ -441,7 +446,7 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
         }
         if (!have_next && sp > 0) {
             --sp;
-            next = (shelf != nullptr && sp < kLaneShelf) ? shelf[sp * DST_WAVE + (int)__lane_id()] : stack[sp];
+            next = (shelf != nullptr && sp < kLaneShelf) ? ((lds_u32)shelf)[sp * DST_WAVE + (int)__lane_id()] : stack[sp];
         }
         ref = (--budget == 0u) ? kWalkDone : next;
     }
