@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path: forward trace + backward re-trace of one ray batch.
 
-Default workload = BASELINE config 3: 1,000,000 surfels in a 10 m room, 1920x1080 pinhole rays, SH degree 3,
+Default workload (config3): 1,000,000 surfels in a 10 m room, 1920x1080 pinhole rays, SH degree 3,
 max_trace_depth 0, fp32, training mode (a_weights atomics on), seed 0, synthetic data.
 A step = one forward launch + one backward launch through the launcher boundary (output allocation and
 zero-initialisation of the gradient buffers included, as in the reference launcher); inputs are resident in HBM.
@@ -24,18 +24,34 @@ for _p in (ROOT, os.path.join(ROOT, "diff-surfel-tracing_amd")):
 
 HBM_PEAK_GBS = 8000.0
 
-# Algorithmic bytes (AUX=2, MID=16, two mid slots, SH3, training): per ray and per evaluated / composited hit.
-FWD_RAY, FWD_PROC, FWD_CON = 204, 40, 208
-BWD_RAY, BWD_PROC, BWD_CON = 272, 40, 764
-PER_SURFEL_INIT = 316   # zero-fill of the gradient buffers (312) and a_weights (4)
+def algorithmic_bytes(aux, slots, sh_degree=3, training=True):
+    """Bytes per ray and per evaluated / composited hit that the path must move whatever the implementation
+    (BVH traffic excluded): (fwd_ray, fwd_proc, fwd_con), (bwd_ray, bwd_proc, bwd_con), per-surfel zero-fill.
+    `aux` channels, `slots` = mid_val slots per ray.  With aux 2, two slots, SH3, training:
+    (204, 40, 208), (272, 40, 764), 316."""
+    mid = 11 + aux + 3
+    sh = 12 * (sh_degree + 1) ** 2
+    fwd = (24 + 4 * (11 + aux + mid * slots), 40, sh + 4 * aux + (8 if training else 0))
+    bwd = (24 + 4 * (11 + aux) + 4 * mid * slots + 4 * (9 + aux) + 24, 40,
+           sh + 4 * aux + 36 + 8 * (16 + aux + 3 * (sh_degree + 1) ** 2))
+    per_surfel = 4 * (3 + 3 + 3 + 3 * (sh_degree + 1) ** 2 + 3 + aux + 1 + 2 + 4 + 9) + 4
+    return fwd, bwd, per_surfel
 
 
 def workloads():
     import dst_scenes as S
     return {
-        "config1": dict(name="cfg1 cube P=10k 128x128 SH3 depth0", scene=lambda: S.scene_cube(10000), rays=lambda: S.rays_cube(128, 128)),
-        "config2": dict(name="cfg2 sphere P=100k 800x800 SH3 depth0", scene=lambda: S.scene_sphere(100000), rays=lambda: S.rays_sphere(800, 800)),
-        "config3": dict(name="cfg3 room P=1M 1920x1080 SH3 depth0", scene=lambda: S.scene_room(1000000), rays=lambda: S.rays_room(1080, 1920)),
+        "config1": dict(name="cfg1 cube P=10k 128x128 SH3 depth0", scene=lambda: S.scene_cube(10000),
+                        rays=lambda: S.rays_cube(128, 128)),
+        "config2": dict(name="cfg2 sphere P=100k 800x800 SH3 depth0", scene=lambda: S.scene_sphere(100000),
+                        rays=lambda: S.rays_sphere(800, 800)),
+        "config3": dict(name="cfg3 room P=1M 1920x1080 SH3 depth0", scene=lambda: S.scene_room(1000000),
+                        rays=lambda: S.rays_room(1080, 1920)),
+        "config4": dict(name="cfg4 room P=500k 1280x720 SH3 aux8 depth2 threshold0.1",
+                        scene=lambda: S.scene_room(500000, aux=8), rays=lambda: S.rays_room(720, 1280),
+                        aux=8, depth=2, threshold=0.1),
+        "config5": dict(name="cfg5 lidar P=2M (1,131072,3) SH3 aux4 depth0", scene=lambda: S.scene_lidar(2000000),
+                        rays=lambda: S.rays_lidar(), aux=4),
     }
 
 
@@ -44,7 +60,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="config3", choices=["config1", "config2", "config3"])
+    ap.add_argument("--workload", default="config3", choices=["config1", "config2", "config3", "config4", "config5"])
     ap.add_argument("--cpu-stride", type=int, default=1, help="CPU baseline traces every n-th pixel row and column")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -70,7 +86,11 @@ def main():
     R, P = H * W, sc_cpu["means3D"].shape[0]
     g = {k: v.to(dev) for k, v in sc_cpu.items()}
     ro, rd = o_cpu.to(dev), d_cpu.to(dev)
-    ug = {k: v.to(dev) for k, v in S.upstream_grads(H, W, 2).items()}
+    aux, depth, threshold = wl.get("aux", 0), wl.get("depth", 0), wl.get("threshold", 0.0)
+    aux_out = aux if aux else 2                 # channels of the aux output (2 when the scene has none)
+    slots = max(1, depth) + 1                   # mid_val slots per ray
+    (FWD_RAY, FWD_PROC, FWD_CON), (BWD_RAY, BWD_PROC, BWD_CON), PER_SURFEL_INIT = algorithmic_bytes(aux_out, slots)
+    ug = {k: v.to(dev) for k, v in S.upstream_grads(H, W, aux_out).items()}
     ug["dist"] = torch.zeros(H, W, 1, device=dev)
     tracer = dst.SurfelTracer()
     ctx = tracer.optix_context
@@ -92,13 +112,13 @@ def main():
     bg = torch.zeros(3, device=dev)
     eye = torch.eye(4, device=dev)
     cam = torch.zeros(3, device=dev)
-    common = (g["vertices"], bg, g["means3D"], g["shs"], 3, e, e, g["opacities"], g["scales"], 1.0, g["rotations"], e,
-              eye, eye, cam, False, False, 0, 0.0)
+    common = (g["vertices"], bg, g["means3D"], g["shs"], 3, e, g.get("others_precomp", e), g["opacities"], g["scales"],
+              1.0, g["rotations"], e, eye, eye, cam, False, False, depth, threshold)
     counters = torch.zeros(2, dtype=torch.int64, device=dev)
 
     def step(fwd_events=None, bwd_events=None, count=False):
         # what the autograd function does: the forward trace records its hit buffers, backward replays them
-        rec = _C.HitRecord(H, W, 1, ctx.record_blocks_per_wave, dev)
+        rec = _C.HitRecord(H, W, max(1, depth), ctx.record_blocks_per_wave, dev)
         out = _C.trace_surfels(ctx, True, True, ro, rd, *common, counters=counters if count else None,
                                events=fwd_events, hit_record=rec)
         grads = _C.trace_surfels_backward(ctx, True, ro, rd, *common, *out[:7], ug["rgb"], ug["dpt"], ug["acc"],
@@ -145,8 +165,10 @@ def main():
         return {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": traffic,
                 "algorithmic_bytes_per_launch": int(a_bytes), "avg_launch_ms": round(ms, 4)}
-    per_kernel = {"forward": roofline_of("forward", "k_trace_fwd<2,true,false>", A_fwd, fwd_ms),
-                  "backward": roofline_of("backward", "k_trace_bwd<2,true,false>", A_bwd, bwd_ms)}
+    aux_max = 2 if aux_out <= 2 else (4 if aux_out <= 4 else 8)
+    mixed = "true" if (depth > 0 or H < 8) else "false"   # kernels with the per-lane walk built in
+    per_kernel = {"forward": roofline_of("forward", "k_trace_fwd<%d,true,%s>" % (aux_max, mixed), A_fwd, fwd_ms),
+                  "backward": roofline_of("backward", "k_trace_bwd<%d,true,false>" % aux_max, A_bwd, bwd_ms)}
     # the dominant kernel is the slower one (the two are within a few per cent of each other on this workload,
     # so both are reported under `roofline_kernels`)
     roofline = per_kernel["backward" if bwd_ms >= fwd_ms else "forward"]
@@ -156,8 +178,8 @@ def main():
         "value": round(rays_per_s, 1), "unit": "rays/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": wl["name"], "surfels": P, "rays": R, "sh_degree": 3, "max_trace_depth": 0,
-                   "training": True, "seed": 0},
+        "config": {"workload": wl["name"], "surfels": P, "rays": R, "sh_degree": 3, "max_trace_depth": depth,
+                   "aux_channels": aux, "training": True, "seed": 0},
         "fwd_kernel_ms": round(fwd_ms, 4), "bwd_kernel_ms": round(bwd_ms, 4),
         "bvh_build_ms": round(build_ms, 4), "bvh_refit_ms": round(refit_ms, 4),
         "hits_evaluated_per_ray": round(n_proc / R, 3), "hits_composited_per_ray": round(n_con / R, 3),
@@ -171,7 +193,8 @@ def main():
         so, sd = o_cpu[::st, ::st].contiguous(), d_cpu[::st, ::st].contiguous()
         n = {k: v.numpy() for k, v in sc_cpu.items()}
         s = O.Scene(so.numpy(), sd.numpy(), n["vertices"], n["faces"], n["means3D"], n["opacities"], n["scales"],
-                    n["rotations"], shs=n["shs"])
+                    n["rotations"], shs=n["shs"], others_precomp=n.get("others_precomp"), max_trace_depth=depth,
+                    specular_threshold=threshold)
         cores = min(O.num_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or O.num_threads()))
         f = O.forward(s, O.HITS_BVH_LEXI, counters=False)
         tf = s.trace_seconds
