@@ -242,6 +242,10 @@ def test_raw_launcher_calls_without_a_record(oracle, tracer):
     ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
     refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
     np.testing.assert_array_equal(fwd[0].cpu().numpy(), ref["rgb"])
+    # hit counts: entries evaluated and hits composited, summed over the rays, are the oracle's exactly
+    counters = torch.zeros(2, dtype=torch.int64, device=dev)
+    binding.trace_surfels(ctx, True, True, o.to(dev), d.to(dev), *common, counters=counters)
+    assert counters.tolist() == [int(ref["n_proc"].sum()), int(ref["n_con"].sum())]
     names = ("ray_o", "ray_d", "means3D", "grads3D", None, "shs", "colors_precomp", None, "opacities", "scales",
              "rotations", None)
     for t, k in zip(bwd, names):
