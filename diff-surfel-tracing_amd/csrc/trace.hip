@@ -717,6 +717,39 @@ struct BounceAcc {
     float C[3], D, N[3], O[AUXM], T;
 };
 
+// The SH colour's derivative with respect to the direction it was evaluated for, contracted with the colour
+// gradient gc (backward.cu:100-165).
+struct LastShHit { int g; F3 gc; bool any; };
+__device__ __forceinline__ F3 sh_direction_gradient(int deg, const float *__restrict__ sh, F3 rd, F3 gc) {
+#pragma clang fp contract(fast)
+    auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
+    F3 ddx = f3(0, 0, 0), ddy = f3(0, 0, 0), ddz = f3(0, 0, 0);
+    const float x = rd.x, y = rd.y, z = rd.z;
+    if (deg > 0) {
+        ddx = -SH1 * S(3);
+        ddy = -SH1 * S(1);
+        ddz = SH1 * S(2);
+        if (deg > 1) {
+            const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+            ddx = ddx + SH2[0] * y * S(4) + SH2[2] * 2.f * -x * S(6) + SH2[3] * z * S(7) + SH2[4] * 2.f * x * S(8);
+            ddy = ddy + SH2[0] * x * S(4) + SH2[1] * z * S(5) + SH2[2] * 2.f * -y * S(6) + SH2[4] * 2.f * -y * S(8);
+            ddz = ddz + SH2[1] * y * S(5) + SH2[2] * 4.f * z * S(6) + SH2[3] * x * S(7);
+            if (deg > 2) {
+                ddx = ddx + (SH3[0] * 6.f * xy) * S(9) + (SH3[1] * yz) * S(10) + (SH3[2] * -2.f * xy) * S(11) +
+                      (SH3[3] * -6.f * xz) * S(12) + (SH3[4] * (-3.f * xx + 4.f * zz - yy)) * S(13) +
+                      (SH3[5] * 2.f * xz) * S(14) + (SH3[6] * 3.f * (xx - yy)) * S(15);
+                ddy = ddy + (SH3[0] * 3.f * (xx - yy)) * S(9) + (SH3[1] * xz) * S(10) +
+                      (SH3[2] * (-3.f * yy + 4.f * zz - xx)) * S(11) + (SH3[3] * -6.f * yz) * S(12) +
+                      (SH3[4] * -2.f * xy) * S(13) + (SH3[5] * -2.f * yz) * S(14) + (SH3[6] * -6.f * xy) * S(15);
+                ddz = ddz + (SH3[1] * xy) * S(10) + (SH3[2] * 8.f * yz) * S(11) +
+                      (SH3[3] * 3.f * (2.f * zz - xx - yy)) * S(12) + (SH3[4] * 8.f * xz) * S(13) +
+                      (SH3[5] * (xx - yy)) * S(14);
+            }
+        }
+    }
+    return f3(dot(ddx, gc), dot(ddy, gc), dot(ddz, gc));
+}
+
 // Gradient of one composited hit (reference backward.cu:528-640 and 201-287, 68-166).
 // Pure gradient algebra: nothing here feeds a decision, so contraction is allowed.
 template <int AUXM>
@@ -726,7 +759,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                                              float q0, float q1, float q2, float q3, float opac, float nsign,
                                              F3 normal, const float (&col)[3], const bool (&neg)[3], F3 ro, F3 rd,
                                              const float *__restrict__ sh, F3 &g_ro, F3 &g_rd,
-                                             const GradSink<AUXM> &sink, bool did) {
+                                             const GradSink<AUXM> &sink, bool did, LastShHit &last) {
 #pragma clang fp contract(fast)
     // gradient algebra only: divisions become multiplications by a hardware reciprocal (1 ulp)
     const float num = 1.0f - alpha, inv_num = __builtin_amdgcn_rcpf(num);
@@ -837,8 +870,6 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
             sink.add(RowLayout<AUXM>::sh0 + 3 * j + 1, basis * gc.y);
             sink.add(RowLayout<AUXM>::sh0 + 3 * j + 2, basis * gc.z);
         };
-        auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
-        F3 ddx = f3(0, 0, 0), ddy = f3(0, 0, 0), ddz = f3(0, 0, 0);
         const float x = rd.x, y = rd.y, z = rd.z;
         float basis[16];
 #pragma unroll
@@ -848,9 +879,6 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
             basis[1] = -SH1 * y;
             basis[2] = SH1 * z;
             basis[3] = -SH1 * x;
-            ddx = -SH1 * S(3);
-            ddy = -SH1 * S(1);
-            ddz = SH1 * S(2);
             if (deg > 1) {
                 const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
                 basis[4] = SH2[0] * xy;
@@ -858,9 +886,6 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                 basis[6] = SH2[2] * (2.f * zz - xx - yy);
                 basis[7] = SH2[3] * xz;
                 basis[8] = SH2[4] * (xx - yy);
-                ddx = ddx + SH2[0] * y * S(4) + SH2[2] * 2.f * -x * S(6) + SH2[3] * z * S(7) + SH2[4] * 2.f * x * S(8);
-                ddy = ddy + SH2[0] * x * S(4) + SH2[1] * z * S(5) + SH2[2] * 2.f * -y * S(6) + SH2[4] * 2.f * -y * S(8);
-                ddz = ddz + SH2[1] * y * S(5) + SH2[2] * 4.f * z * S(6) + SH2[3] * x * S(7);
                 if (deg > 2) {
                     basis[9] = SH3[0] * y * (3.f * xx - yy);
                     basis[10] = SH3[1] * xy * z;
@@ -869,22 +894,19 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                     basis[13] = SH3[4] * x * (4.f * zz - xx - yy);
                     basis[14] = SH3[5] * z * (xx - yy);
                     basis[15] = SH3[6] * x * (xx - 3.f * yy);
-                    ddx = ddx + (SH3[0] * 6.f * xy) * S(9) + (SH3[1] * yz) * S(10) + (SH3[2] * -2.f * xy) * S(11) +
-                          (SH3[3] * -6.f * xz) * S(12) + (SH3[4] * (-3.f * xx + 4.f * zz - yy)) * S(13) +
-                          (SH3[5] * 2.f * xz) * S(14) + (SH3[6] * 3.f * (xx - yy)) * S(15);
-                    ddy = ddy + (SH3[0] * 3.f * (xx - yy)) * S(9) + (SH3[1] * xz) * S(10) +
-                          (SH3[2] * (-3.f * yy + 4.f * zz - xx)) * S(11) + (SH3[3] * -6.f * yz) * S(12) +
-                          (SH3[4] * -2.f * xy) * S(13) + (SH3[5] * -2.f * yz) * S(14) + (SH3[6] * -6.f * xy) * S(15);
-                    ddz = ddz + (SH3[1] * xy) * S(10) + (SH3[2] * 8.f * yz) * S(11) +
-                          (SH3[3] * 3.f * (2.f * zz - xx - yy)) * S(12) + (SH3[4] * 8.f * xz) * S(13) +
-                          (SH3[5] * (xx - yy)) * S(14);
                 }
             }
         }
 #pragma unroll
         for (int j = 0; j < 16; ++j) put(j, basis[j]);
         sink.finish(RowLayout<AUXM>::cols);
-        if (did) g_rd = f3(dot(ddx, gc), dot(ddy, gc), dot(ddz, gc));
+        // The reference overwrites the ray-direction gradient with the SH term at every hit (backward.cu:165), so
+        // only the last composited hit's term survives: remember it, walk_bounce computes it once per bounce.
+        if (did) {
+            last.g = g;
+            last.gc = gc;
+            last.any = true;
+        }
     }
 }
 
@@ -979,6 +1001,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     F3 ot = ro;
     bool live = lane_on;
     KBuf buf;
+    LastShHit last_sh = {0, f3(0, 0, 0), false};
     // kernels built without the per-lane walk (MIXED false) take every wave as a packet
     const bool as_packet = (!MIXED || (REC && BWD)) ? true : rays_run_together(ro, rd, lane_on, max_abs);
     uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
@@ -1144,7 +1167,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                      ws.nodes += __popcll(wave_ballot(did && sink.own_slot < 0)); ws.leaves += __popcll(wave_ballot(sink.stray));
                      ws.leaf_any += __popcll(wave_ballot(did));)
                 hit_backward<AUXM>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
-                                   q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did);
+                                   q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did, last_sh);
                 STAT(ws.t_hb += __builtin_readcyclecounter() - d1;)
             }
         }
@@ -1170,6 +1193,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         }
     }
+    if (BWD && p.colors_precomp == nullptr && last_sh.any)
+        g_rd = sh_direction_gradient(p.D, p.shs + (size_t)last_sh.g * p.M * 3, rd, last_sh.gc);
     run.T = Tp;
 }
 
