@@ -125,3 +125,17 @@ def test_scene_generators_have_the_documented_shapes():
     assert o.shape == d.shape == (1, 128, 3)
     a, b = S.scene_cube(P=32, seed=7), S.scene_cube(P=32, seed=7)
     assert all(torch.equal(a[k], b[k]) for k in a)   # seeded: identical on every machine
+
+
+def test_bench_byte_formula_reproduces_the_documented_constants():
+    """bench.py's general byte formula at the reference constants (aux 2, two mid slots, SH3, training) is
+    204 + 40 n_proc + 208 n_con forward, 272 + 40 n_proc + 764 n_con backward, 316 per surfel."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(os.path.dirname(__file__), "..", "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert bench.algorithmic_bytes(2, 2) == ((204, 40, 208), (272, 40, 764), 316)
+    fwd8, bwd8, per8 = bench.algorithmic_bytes(8, 3)            # config 4: aux 8, three mid slots
+    assert fwd8[0] == 24 + 4 * (11 + 8 + 22 * 3) and fwd8[2] == 192 + 32 + 8 and per8 == 316 + 4 * 6
+    assert sorted(bench.workloads()) == ["config1", "config2", "config3", "config4", "config5"]
