@@ -118,11 +118,12 @@ def main():
 
     def step(fwd_events=None, bwd_events=None, count=False):
         # what the autograd function does: the forward trace records its hit buffers, backward replays them
-        rec = _C.HitRecord(H, W, max(1, depth), ctx.record_blocks_per_wave, dev)
+        rec = ctx.acquire_record(H, W, max(1, depth), dev)
         out = _C.trace_surfels(ctx, True, True, ro, rd, *common, counters=counters if count else None,
                                events=fwd_events, hit_record=rec)
         grads = _C.trace_surfels_backward(ctx, True, ro, rd, *common, *out[:7], ug["rgb"], ug["dpt"], ug["acc"],
                                           ug["norm"], ug["dist"], ug["aux"], events=bwd_events, hit_record=rec)
+        ctx.release_record(rec)
         return out, grads
 
     for _ in range(args.warmup):

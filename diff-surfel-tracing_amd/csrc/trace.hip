@@ -2,7 +2,7 @@
 //
 // One wavefront (64 lanes) carries an 8x8 tile of rays as a PACKET: the BVH walk is wave-uniform
 // (node and leaf records are fetched once per wave through the scalar path, the traversal stack
-// is a single VGPR indexed by lane), every lane tests its own ray against the shared node / quad,
+// is two VGPRs indexed by lane), every lane tests its own ray against the shared node / quad,
 // and each lane keeps its own 16-entry nearest-hit buffer in registers.  Replaces the raygen /
 // any-hit programs of the reference (optix_tracer/forward.cu, optix_tracer/backward.cu).
 //
@@ -913,7 +913,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
 // ---- hit record: the forward trace can store every chunk's hit buffer, the backward trace then replays
 // them instead of walking the BVH again.  Layout of the caller's buffer, in 8-byte words:
 //   [0] blocks requested so far (the forward kernel counts on past the capacity, which is how overflow shows)
-//   [1] unused
+//   [1] chains that a replay found broken (stays 0 for a record written by a forward trace with a zeroed header)
 //   [2 ...) directory: one uint32 per (wave, bounce slot) = 1 + first block of that wave's bounce, 0 = none
 //   then `capacity` blocks of kRecBlockWords words: 16x64 entries ([slot][lane]), 64 uint32 counts, next+1.
 constexpr uint32_t kRecBlockWords = kChunk * DST_WAVE + DST_WAVE / 2 + 8;
@@ -1023,7 +1023,11 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         const uint32_t lane_ = __lane_id();
         if (REC && BWD) {
             rec_block = rec_open(rv, rec_pos, cnt);
-            if (rec_block == nullptr) { live = false; break; }   // cannot happen with a complete record
+            if (rec_block == nullptr) {   // cannot happen with a complete record: count it where the caller can see it
+                if (lane_ == 0) atomicAdd((unsigned long long *)(rv.base + 1), 1ull);
+                live = false;
+                break;
+            }
         } else {
             kbuf_reset(buf);
             packet_knn<MIXED, MIXED && !BWD>(acc, max_abs, ot, rd, live, buf, cnt, as_packet WSP);
@@ -1233,6 +1237,13 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     __shared__ float s_stage[BWD ? kWavesPerBlock * kStageWords : 1];
     uint32_t *tab_keys = s_keys;
     float *tab_rows = s_rows;
+    // Backward with a hit record: the launcher starts the replaying kernel and the re-tracing kernel one after
+    // the other, and word 0 of the record (blocks the forward trace asked for) decides on the device which of
+    // the two does the work: the host never has to wait for the forward trace to learn whether its record is complete.
+    if (BWD && p.hit_record != nullptr) {
+        const bool complete = p.hit_record[0] <= (uint64_t)p.hit_record_blocks;
+        if (REC != complete) return;
+    }
     if (BWD) {
         table_clear_keys<AUXM>(s_keys);
         for (int k = threadIdx.x; k < kTableRows * RowLayout<AUXM>::stride; k += kWavesPerBlock * DST_WAVE)
@@ -1555,8 +1566,8 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     acc.root = dst_root_ref(ctx->n_leaves);
     const bool rec = p.hit_record != nullptr;
     if (backward) {
-        if (rec) launch<true, true>(p, acc, t, stream);
-        else launch<true, false>(p, acc, t, stream);
+        if (rec) launch<true, true>(p, acc, t, stream);   // does the work if the record is complete,
+        launch<true, false>(p, acc, t, stream);           // else this one does (it returns at once otherwise)
     } else {
         if (rec) launch<false, true>(p, acc, t, stream);
         else launch<false, false>(p, acc, t, stream);

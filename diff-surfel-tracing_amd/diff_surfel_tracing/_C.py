@@ -108,29 +108,71 @@ def _ptr(t):
 
 class HitRecord:
     """Device buffer in which a forward trace stores its per-chunk hit buffers so that the backward trace can
-    replay them instead of walking the BVH again (see `hit_record` in include/dst_api.h)."""
+    replay them instead of walking the BVH again (see `hit_record` in include/dst_api.h).  `storage` is a
+    caller- or pool-owned int64 tensor that is at least `words_needed(...)` long."""
 
-    def __init__(self, H, W, mtd_alloc, blocks_per_wave, device):
+    @staticmethod
+    def layout(H, W, mtd_alloc, blocks_per_wave):
+        """(words of the whole buffer, header words, blocks, waves) for an (H,W) ray grid."""
         header, waves = C.c_uint64(0), C.c_uint32(0)
         lib = load_library()
         lib.dst_hit_record_layout(H, W, mtd_alloc, 0, C.byref(header), C.byref(waves))
-        self.n_waves = max(1, waves.value)
-        self.blocks = max(1, int(self.n_waves * blocks_per_wave) + 1)
-        words = lib.dst_hit_record_layout(H, W, mtd_alloc, self.blocks, None, None)
-        self.words = torch.empty(words, dtype=torch.int64, device=device)
-        self.words[: header.value].zero_()
+        n_waves = max(1, waves.value)
+        blocks = max(1, int(n_waves * blocks_per_wave) + 1)
+        words = lib.dst_hit_record_layout(H, W, mtd_alloc, blocks, None, None)
+        return int(words), int(header.value), blocks, n_waves
+
+    def __init__(self, H, W, mtd_alloc, blocks_per_wave, device, storage=None):
+        words, header, self.blocks, self.n_waves = self.layout(H, W, mtd_alloc, blocks_per_wave)
+        if storage is None:
+            storage = torch.empty(words, dtype=torch.int64, device=device)
+        elif storage.numel() < words or storage.dtype != torch.int64 or not storage.is_cuda:
+            raise RuntimeError("hit record storage must be a CUDA int64 tensor of at least %d elements" % words)
+        self.words = storage
+        self.words[:header].zero_()
+        self._asked_host = None
+        self._asked_event = None
+
+    def note_request(self):
+        """Stream-ordered, non-blocking copy of word 0 (blocks the forward trace asked for) to pinned host
+        memory; `asked()` reads it once the copy has happened."""
+        self._asked_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+        self._asked_host.copy_(self.words[:1], non_blocking=True)
+        self._asked_event = torch.cuda.Event()
+        self._asked_event.record()
+
+    def asked(self, wait=False):
+        """Blocks requested by the forward trace, or None while that is not known yet (never waits unless told to)."""
+        if self._asked_event is None:
+            return int(self.words[0].item()) if wait else None
+        if wait:
+            self._asked_event.synchronize()
+        elif not self._asked_event.query():
+            return None
+        return int(self._asked_host[0])
 
     def requested_blocks(self):
         """Blocks the forward trace asked for (waits for it to finish)."""
-        return int(self.words[0].item())
+        return self.asked(wait=True)
 
     def complete(self):
         return self.requested_blocks() <= self.blocks
 
+    def broken_chains(self):
+        """Chains a replaying backward trace found broken (waits); 0 for every record a forward trace wrote."""
+        return int(self.words[1].item())
+
 
 class OptiXStateWrapper:
     """Owner of the acceleration structure; keeps the reference's class name (ext.cpp:8) so callers need not
-    change.  `pkg_dir` was where the reference looked for its PTX files and is ignored."""
+    change.  `pkg_dir` was where the reference looked for its PTX files and is ignored.
+
+    Also owns the hit-record buffers of the autograd path: a small pool that forward calls draw from and
+    backward calls return to (no allocation per call once warm), bounded by `record_max_bytes` per record; a
+    record that would be larger, or whose allocation fails, is simply not made and the backward pass walks the
+    BVH again."""
+
+    RECORD_POOL_SIZE = 4
 
     def __init__(self, pkg_dir=None):
         lib = load_library()
@@ -142,6 +184,60 @@ class OptiXStateWrapper:
         self.device = torch.cuda.current_device()
         self.num_surfels = 0
         self.record_blocks_per_wave = 6.0   # sizing estimate for hit records, raised when a record overflows
+        self.record_max_bytes = 8 << 30     # no record larger than this is made (backward then re-traces)
+        self.record_wanted = True           # set by the autograd wrapper for the call that follows
+        self._record_pool = []              # free storages (int64 tensors)
+        self._record_fixed = False          # True: only caller-provided storage is used, nothing is allocated
+        self._record_watch = []             # records whose request count has not been read yet
+
+    # ---- hit-record storage ---------------------------------------------------------------------------
+    def use_record_storage(self, storage):
+        """Use this caller-owned int64 CUDA tensor (and nothing else) for hit records; None returns to the
+        pool.  One record is live at a time with a fixed storage: a forward call that finds it taken, or too
+        small (HitRecord.layout gives the size), makes no record."""
+        self._record_pool = [] if storage is None else [storage]
+        self._record_fixed = storage is not None
+
+    def update_record_estimate(self):
+        """Raise the sizing estimate from records whose forward trace has finished; never waits."""
+        still = []
+        for rec in self._record_watch:
+            asked = rec.asked()
+            if asked is None:
+                still.append(rec)
+            else:
+                self.record_blocks_per_wave = max(self.record_blocks_per_wave, 1.25 * asked / rec.n_waves)
+        self._record_watch = still[-8:]
+
+    def acquire_record(self, H, W, mtd_alloc, device):
+        self.update_record_estimate()
+        words = HitRecord.layout(H, W, mtd_alloc, self.record_blocks_per_wave)[0]
+        if 8 * words > self.record_max_bytes:
+            return None
+        device = torch.device(device)
+        if device.index is None:
+            device = torch.device(device.type, torch.cuda.current_device())
+        fit = [t for t in self._record_pool if t.numel() >= words and t.device == device]
+        storage = None
+        if fit:
+            storage = min(fit, key=lambda t: t.numel())
+            self._record_pool = [t for t in self._record_pool if t is not storage]
+        elif self._record_fixed:
+            return None
+        else:
+            try:
+                storage = torch.empty(words + words // 8, dtype=torch.int64, device=device)
+            except torch.OutOfMemoryError:
+                return None
+        return HitRecord(H, W, mtd_alloc, self.record_blocks_per_wave, device, storage=storage)
+
+    def release_record(self, rec):
+        if rec is None or rec.words is None:
+            return
+        self._record_pool.append(rec.words)
+        rec.words = None
+        if not self._record_fixed and len(self._record_pool) > self.RECORD_POOL_SIZE:
+            self._record_pool.remove(min(self._record_pool, key=lambda t: t.numel()))
 
     def accel_info(self):
         info = DstAccelInfo()
@@ -235,6 +331,9 @@ def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, backg
     _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))
     if events is not None:
         events[1].record()
+    if hit_record is not None:
+        hit_record.note_request()
+        ctx._record_watch.append(hit_record)
     del keep
     return out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights
 
@@ -281,11 +380,9 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
     p.dL_dopacities, p.dL_dscales, p.dL_drotations = (dL_dopacities.data_ptr(), dL_dscales.data_ptr(),
                                                       dL_drotations.data_ptr())
     if hit_record is not None:
-        # replay only a complete record; an overflowed one means re-tracing (and a larger estimate next time)
-        asked = hit_record.requested_blocks()
-        ctx.record_blocks_per_wave = max(ctx.record_blocks_per_wave, 1.25 * asked / hit_record.n_waves)
-        if asked <= hit_record.blocks:
-            p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
+        # the kernels decide on the device whether the record is complete (replay) or not (walk the BVH again):
+        # nothing here waits for the forward trace
+        p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
     p.counters = _ptr(counters)
     if events is not None:
         events[0].record()

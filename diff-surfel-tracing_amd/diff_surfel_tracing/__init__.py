@@ -62,13 +62,19 @@ class _TraceSurfels(torch.autograd.Function):
         args = (optix_context, training, start_from_first, ray_o, ray_d, vertices, s.bg, means3D, shs, s.sh_degree,
                 colors_precomp, others_precomp, opacities, scales, s.scale_modifier, rotations,
                 cov3Ds_precomp) + _settings_args(s)
-        # when a backward pass will follow, the forward trace records its hit buffers for it
+        # when a backward pass will follow, the forward trace records its hit buffers for it; the wrapper below
+        # says whether one can follow (gradient mode is always off in here, and needs_input_grad stays set
+        # under torch.no_grad())
         record = None
-        if any(ctx.needs_input_grad) and ray_o.dim() == 3 and ray_o.numel() > 0:
-            record = _C.HitRecord(ray_o.size(0), ray_o.size(1), max(_C.DEFAULT_MAX_TRACE_DEPTH, s.max_trace_depth),
-                                  optix_context.record_blocks_per_wave, ray_o.device)
-        out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights = _guarded(
-            lambda *a: _C.trace_surfels(*a, hit_record=record), args, s.debug, "snapshot_fw.dump", "forward")
+        if optix_context.record_wanted and any(ctx.needs_input_grad) and ray_o.dim() == 3 and ray_o.numel() > 0:
+            record = optix_context.acquire_record(ray_o.size(0), ray_o.size(1),
+                                                  max(_C.DEFAULT_MAX_TRACE_DEPTH, s.max_trace_depth), ray_o.device)
+        try:
+            out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights = _guarded(
+                lambda *a: _C.trace_surfels(*a, hit_record=record), args, s.debug, "snapshot_fw.dump", "forward")
+        except Exception:
+            optix_context.release_record(record)
+            raise
         ctx.hit_record = record
 
         ctx.tracer_settings = s
@@ -92,9 +98,16 @@ class _TraceSurfels(torch.autograd.Function):
                 cov3Ds_precomp) + _settings_args(s) + (
                     out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val,
                     grad_out_rgb, grad_out_dpt, grad_out_acc, grad_out_norm, grad_out_dist, grad_out_aux)
-        (g_ray_o, g_ray_d, g_means3D, g_grads3D, _g_grads3D_abs, g_shs, g_colors, g_others, g_opacities, g_scales,
-         g_rotations, g_cov3Ds) = _guarded(lambda *a: _C.trace_surfels_backward(*a, hit_record=ctx.hit_record), args,
-                                           s.debug, "snapshot_bw.dump", "backward")
+        record = ctx.hit_record if (ctx.hit_record is not None and ctx.hit_record.words is not None) else None
+        try:
+            (g_ray_o, g_ray_d, g_means3D, g_grads3D, _g_grads3D_abs, g_shs, g_colors, g_others, g_opacities,
+             g_scales, g_rotations, g_cov3Ds) = _guarded(
+                 lambda *a: _C.trace_surfels_backward(*a, hit_record=record), args, s.debug, "snapshot_bw.dump",
+                 "backward")
+        finally:
+            # the storage goes back to the pool (stream-ordered reuse); a second backward through the same graph
+            # (retain_graph) walks the BVH again
+            ctx.optix_context.release_record(record)
 
         def like(grad, inp):  # an absent optional input (empty placeholder tensor) gets no gradient
             return grad if inp.numel() != 0 else None
@@ -107,6 +120,11 @@ class _TraceSurfels(torch.autograd.Function):
 
 def trace_surfels(optix_context, training, start_from_first, ray_o, ray_d, vertices, means3D, grads3D, shs,
                   colors_precomp, others_precomp, opacities, scales, rotations, cov3Ds_precomp, tracer_settings):
+    # a hit record only pays off when a backward pass can follow: not under torch.no_grad(), not for inputs
+    # without gradients (the usual evaluation loop renders nn.Parameter tensors under no_grad)
+    optix_context.record_wanted = torch.is_grad_enabled() and any(
+        isinstance(t, torch.Tensor) and t.requires_grad
+        for t in (ray_o, ray_d, means3D, grads3D, shs, colors_precomp, others_precomp, opacities, scales, rotations))
     return _TraceSurfels.apply(optix_context, training, start_from_first, ray_o, ray_d, vertices, means3D, grads3D,
                                shs, colors_precomp, others_precomp, opacities, scales, rotations, cov3Ds_precomp,
                                tracer_settings)

@@ -78,11 +78,14 @@ typedef struct DstParams {
     /* optional forward statistics: counters[0] += entries evaluated, counters[1] += hits composited */
     unsigned long long *counters;
     /* optional hit record (no counterpart in the reference): when non-NULL the forward trace stores every
-     * chunk's 16-entry hit buffer in it, and a backward trace given the same, complete record replays the
-     * buffers instead of walking the BVH again (same results, no traversal).  Device memory, 8-byte aligned,
-     * sized with dst_hit_record_layout(); the caller zero-fills the first header_words words before the
-     * forward call.  Word 0 then holds the number of blocks the forward trace asked for: if that exceeds
-     * hit_record_blocks the record is incomplete and must not be passed to the backward call. */
+     * chunk's 16-entry hit buffer in it, and a backward trace given the same record replays the buffers
+     * instead of walking the BVH again (same results, no traversal).  Device memory, 8-byte aligned, sized
+     * with dst_hit_record_layout(); the caller zero-fills the first header_words words before the forward
+     * call.  Word 0 then holds the number of blocks the forward trace asked for.  If that exceeds
+     * hit_record_blocks the record is incomplete: the backward trace sees this ON THE DEVICE and walks the BVH
+     * again instead (the host need not look at the record between the two calls; it may read word 0 later to
+     * size the next record).  Word 1 counts chains a replay found broken: it stays 0 unless the buffer was
+     * not written by a forward trace with the same grid, depth and a zeroed header. */
     uint64_t *hit_record;
     uint32_t hit_record_blocks;
     uint32_t reserved0;

@@ -139,3 +139,51 @@ def test_bench_byte_formula_reproduces_the_documented_constants():
     fwd8, bwd8, per8 = bench.algorithmic_bytes(8, 3)            # config 4: aux 8, three mid slots
     assert fwd8[0] == 24 + 4 * (11 + 8 + 22 * 3) and fwd8[2] == 192 + 32 + 8 and per8 == 316 + 4 * 6
     assert sorted(bench.workloads()) == ["config1", "config2", "config3", "config4", "config5"]
+
+
+class _FakeContext:
+    """Stands in for OptiXStateWrapper in host tests: remembers whether a hit record was asked for."""
+
+    def __init__(self):
+        self.record_wanted = True
+        self.acquired = 0
+        self.released = 0
+
+    def acquire_record(self, H, W, mtd_alloc, device):
+        self.acquired += 1
+        return None   # "too large": the backward pass would walk the BVH again
+
+    def release_record(self, rec):
+        self.released += 1
+
+
+def test_no_hit_record_is_made_when_no_backward_can_follow(monkeypatch):
+    """Evaluation loops render nn.Parameter tensors under torch.no_grad(): `needs_input_grad` is still set inside
+    the autograd function then, so the wrapper must look at the gradient mode before the call."""
+    import diff_surfel_tracing as dst
+    from diff_surfel_tracing import _C
+
+    def fake_trace(ctx, training, sff, ray_o, *rest, hit_record=None):
+        H, W = ray_o.shape[:2]
+        z = lambda c: torch.zeros(H, W, c)  # noqa: E731
+        return z(3), z(1), z(1), z(3), z(3), z(2), z(32), None
+
+    monkeypatch.setattr(_C, "trace_surfels", fake_trace)
+    eye = torch.eye(4)
+    st = dst.SurfelTracingSettings(4, 4, 1.0, 1.0, torch.zeros(3), 1.0, eye, eye, 3, torch.zeros(3), False, False)
+    P = 5
+    means = torch.nn.Parameter(torch.zeros(P, 3))
+    args = lambda ctx: (ctx, True, True, torch.zeros(4, 4, 3), torch.zeros(4, 4, 3), torch.zeros(4 * P, 3), means,  # noqa: E731
+                        torch.zeros(P, 3), torch.zeros(P, 16, 3), torch.empty(0), torch.empty(0),
+                        torch.zeros(P, 1), torch.ones(P, 2), torch.zeros(P, 4), torch.empty(0), st)
+    ctx = _FakeContext()
+    with torch.no_grad():
+        dst.trace_surfels(*args(ctx))
+    assert ctx.acquired == 0
+    dst.trace_surfels(*args(ctx))
+    assert ctx.acquired == 1
+    ctx2 = _FakeContext()
+    plain = list(args(ctx2))
+    plain[6] = torch.zeros(P, 3)       # no input asks for a gradient
+    dst.trace_surfels(*plain)
+    assert ctx2.acquired == 0
