@@ -54,6 +54,10 @@ dst_ctx *dst_create(void) {
         delete ctx;
         return nullptr;
     }
+    if (dst_static_scratch_init(ctx) != DST_OK) {   // once per device, with that device current
+        delete ctx;
+        return nullptr;
+    }
     return ctx;
 }
 
@@ -83,8 +87,28 @@ int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, co
         if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "refit (rebuild=False) before any build");
         if (P != ctx->n_leaves)
             return dst_fail(ctx, DST_E_TOPOLOGY, "refit (rebuild=False) with a different number of surfels");
+        if (n_vertices < ctx->built_vertices)
+            return dst_fail(ctx, DST_E_TOPOLOGY, "refit (rebuild=False) with fewer vertices than the build indexed");
     }
     return dst_lbvh_build(ctx, vertices, n_vertices, triangles, P, rebuild != 0, (hipStream_t)stream);
+}
+
+int dst_refit_accel_static(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, void *stream) {
+    if (!ctx) return DST_E_INVALID;
+    if (!vertices) return dst_fail(ctx, DST_E_INVALID, "vertices must have dimensions (num_vertices, 3)");
+    if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "refit before any build");
+    if (ctx->n_leaves > DST_STATIC_REFIT_MAX_SURFELS)
+        return dst_fail(ctx, DST_E_UNSUPPORTED, "dst_refit_accel_static holds scratch for at most " +
+                                                    std::to_string(DST_STATIC_REFIT_MAX_SURFELS) + " surfels (" +
+                                                    std::to_string(ctx->n_leaves) + " in the structure)");
+    if (n_vertices < ctx->built_vertices)
+        return dst_fail(ctx, DST_E_TOPOLOGY, "refit with fewer vertices than the build indexed");
+    int dev = -1;
+    DST_HIP(ctx, hipGetDevice(&dev));
+    if (dev != ctx->device) return dst_fail(ctx, DST_E_INVALID, "the context belongs to another device");
+    uint32_t *scratch = dst_static_scratch(ctx);
+    if (!scratch) return dst_fail(ctx, DST_E_DEVICE, "static scratch was not set up on this device");
+    return dst_lbvh_build(ctx, vertices, n_vertices, nullptr, ctx->n_leaves, false, (hipStream_t)stream, scratch);
 }
 
 int dst_trace_forward(dst_ctx *ctx, const DstParams *p, void *stream) {

@@ -72,6 +72,7 @@ struct dst_ctx {
     uint32_t n_leaves = 0;      // surfels in the current structure
     uint32_t capacity = 0;      // surfels the buffers can hold
     bool built = false;
+    uint32_t built_vertices = 0;   // rows of the vertex buffer the stored quad ids were validated against
     uint32_t builds = 0, refits = 0;
     DstNode *nodes = nullptr;
     DstWideNode *wide = nullptr;
@@ -94,8 +95,12 @@ static inline uint32_t dst_root_ref(uint32_t n_leaves) {
 }
 
 // lbvh.hip
+// `fit_flags`: arrival counters of the bottom-up fit (one per surfel); nullptr = the context's own.
 int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
-                   uint32_t n_surfels, bool rebuild, hipStream_t stream);
+                   uint32_t n_surfels, bool rebuild, hipStream_t stream, uint32_t *fit_flags = nullptr);
+// Per-device address of the static scratch array (set up once per device by dst_create).
+int dst_static_scratch_init(dst_ctx *ctx);
+uint32_t *dst_static_scratch(const dst_ctx *ctx);
 void dst_lbvh_free(dst_ctx *ctx);
 // trace.hip
 int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream);

@@ -478,7 +478,29 @@ int ensure_capacity(dst_ctx *ctx, uint32_t P) {
     return DST_OK;
 }
 
+// Scratch of dst_refit_accel_static: the arrival counters of the bottom-up fit, one per surfel.  One copy per
+// GPU, held until the process ends; host code reaches it only through the address hipGetSymbolAddress returns
+// on that GPU (the array's name is not a device address on the host side).
+__device__ __align__(256) uint32_t g_refit_scratch[DST_STATIC_REFIT_MAX_SURFELS];
+constexpr int kMaxDevices = 64;
+uint32_t *g_refit_scratch_ptr[kMaxDevices] = {};
+
 }  // namespace
+
+int dst_static_scratch_init(dst_ctx *ctx) {
+    const int dev = ctx->device;
+    if (dev < 0 || dev >= kMaxDevices) return dst_fail(ctx, DST_E_UNSUPPORTED, "device ordinal beyond 63");
+    if (g_refit_scratch_ptr[dev] != nullptr) return DST_OK;
+    uint32_t *ptr = nullptr;
+    DST_HIP(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(g_refit_scratch)));
+    if (ptr == nullptr) return dst_fail(ctx, DST_E_DEVICE, "hipGetSymbolAddress returned no address");
+    g_refit_scratch_ptr[dev] = ptr;
+    return DST_OK;
+}
+
+uint32_t *dst_static_scratch(const dst_ctx *ctx) {
+    return (ctx->device >= 0 && ctx->device < kMaxDevices) ? g_refit_scratch_ptr[ctx->device] : nullptr;
+}
 
 void dst_lbvh_free(dst_ctx *ctx) {
     auto rel = [](auto *&p) {
@@ -504,13 +526,16 @@ void dst_lbvh_free(dst_ctx *ctx) {
 }
 
 int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles, uint32_t P,
-                   bool rebuild, hipStream_t stream) {
+                   bool rebuild, hipStream_t stream, uint32_t *fit_flags) {
     if (rebuild) {
         ctx->built = false;
         int rc = ensure_capacity(ctx, P);
         if (rc) return rc;
         ctx->n_leaves = P;
     }
+    if (fit_flags == nullptr) fit_flags = ctx->flags;   // after ensure_capacity: a first build allocates them there
+    if (fit_flags == nullptr || ctx->nodes == nullptr || ctx->leaves == nullptr || ctx->vals[0] == nullptr)
+        return dst_fail(ctx, DST_E_DEVICE, "acceleration structure buffers are not allocated");
     const uint32_t n = P;
     int4 *quad_ids = reinterpret_cast<int4 *>(ctx->quad_ids);
     float4 *centroids = reinterpret_cast<float4 *>(ctx->centroids);
@@ -549,9 +574,9 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     }
     hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0], ctx->leaves,
                        n);
-    hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->flags, 0u, n);
+    hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, fit_flags, 0u, n);
     hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
-                       ctx->flags, ctx->leaves, n);
+                       fit_flags, ctx->leaves, n);
     if (n > DST_GROUP)
         hipLaunchKernelGGL(k_widen, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, ctx->wide, n - 1);
     DST_HIP(ctx, hipGetLastError());
@@ -567,6 +592,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
             ctx->scene_hi[a] = ord2f(ctx->bounds_host->hi[a]);
         }
         std::memcpy(&ctx->max_abs, &ctx->bounds_host->max_abs, 4);
+        ctx->built_vertices = n_vertices;
         ctx->built = true;
         ctx->builds++;
     } else {

@@ -45,7 +45,7 @@ class DstAccelInfo(C.Structure):
 
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
            "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params",
-           "dst_hit_record_layout")
+           "dst_hit_record_layout", "dst_refit_accel_static")
 
 _lib = None
 
@@ -64,6 +64,7 @@ def load_library():
     L.dst_destroy.restype = None
     L.dst_destroy.argtypes = [C.c_void_p]
     L.dst_build_accel.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_int, C.c_void_p]
+    L.dst_refit_accel_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p]
     L.dst_trace_forward.argtypes = [C.c_void_p, C.POINTER(DstParams), C.c_void_p]
     L.dst_trace_backward.argtypes = [C.c_void_p, C.POINTER(DstParams), C.c_void_p]
     L.dst_last_error.restype = C.c_char_p

@@ -37,6 +37,7 @@ enum {
 
 #define DST_MAX_AUX 8        /* auxiliary channels per surfel (reference AUX_CHANNELS = 2) */
 #define DST_MAX_TRACE_DEPTH 3 /* bounces after the primary ray (reference MAX_TRACE_DEPTH = 1) */
+#define DST_STATIC_REFIT_MAX_SURFELS (1u << 21) /* largest structure dst_refit_accel_static serves */
 
 /* Opaque tracer state: owns the acceleration structure and its scratch.
  * Replaces OptiXStateWrapper (optix_tracer/optix_wrapper.h:25-52). */
@@ -128,6 +129,17 @@ void dst_destroy(dst_ctx *ctx);
  * Replaces BuildAccelerationStructure (trace_surfels.cpp:36-159). */
 int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
                     uint32_t n_triangles, int rebuild, void *stream);
+
+/* Refit that allocates nothing: dst_build_accel with rebuild == 0, except that the scratch of the refit
+ * kernels (one arrival counter per surfel for the bottom-up box fit) is a fixed array inside the library,
+ * 4 bytes x DST_STATIC_REFIT_MAX_SURFELS = 8 MiB, which every GPU the library runs on holds until the process
+ * ends.  No counterpart in the reference; it is for callers that cannot allocate device memory: code under
+ * stream capture, tight per-frame serving loops, harnesses that forbid it.  Calls no hipMalloc / hipFree.
+ * A structure of more than DST_STATIC_REFIT_MAX_SURFELS surfels is rejected with DST_E_UNSUPPORTED.  All
+ * contexts on one GPU share the array: calls that overlap on one GPU (different streams or threads) race;
+ * calls ordered on one stream do not (the counters are cleared by a fill kernel at the start of each call).
+ * Stream-ordered, no wait; same results as dst_build_accel(..., rebuild = 0, ...). */
+int dst_refit_accel_static(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, void *stream);
 
 /* Forward trace: fills out_* and mid_val, accumulates a_weights.
  * Replaces TraceSurfelsCUDA (trace_surfels.cpp:162-304); stream-ordered, no wait. */
