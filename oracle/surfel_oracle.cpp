@@ -85,18 +85,26 @@ constexpr float C2[5] = {1.0925484305920792f, -1.0925484305920792f, 0.3153915652
 constexpr float C3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.4570457994644658f, 0.3731763325901154f,
                          -0.4570457994644658f, 1.445305721320277f, -0.5900435899266435f};
 
-struct V3 { float x, y, z; };
+// V3T<float> carries every decision; the gradient algebra is written once for float (the restatement of the
+// reference, which is what the GPU path is compared with) and for double (same formulas, same fp32 inputs and
+// decisions: shows how much of a float gradient value is rounding of an ill-conditioned formula).
+template <typename T> struct V3T { T x, y, z; };
+using V3 = V3T<float>;
+template <typename T> inline V3T<T> v3t(T x, T y, T z) { return V3T<T>{x, y, z}; }
 inline V3 v3(float x, float y, float z) { return V3{x, y, z}; }
 inline V3 ld3(const float *p) { return V3{p[0], p[1], p[2]}; }
-inline V3 operator+(V3 a, V3 b) { return V3{a.x + b.x, a.y + b.y, a.z + b.z}; }
-inline V3 operator-(V3 a, V3 b) { return V3{a.x - b.x, a.y - b.y, a.z - b.z}; }
-inline V3 operator-(V3 a) { return V3{-a.x, -a.y, -a.z}; }
-inline V3 operator*(V3 a, float s) { return V3{a.x * s, a.y * s, a.z * s}; }
-inline V3 operator*(float s, V3 a) { return V3{s * a.x, s * a.y, s * a.z}; }
-inline V3 operator/(V3 a, float s) { return V3{a.x / s, a.y / s, a.z / s}; }
-inline float dot(V3 a, V3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
-inline V3 cross(V3 a, V3 b) { return V3{a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x}; }
-inline float len(V3 a) { return std::sqrt(dot(a, a)); }
+template <typename T> inline V3T<T> cast3(V3 a) { return V3T<T>{(T)a.x, (T)a.y, (T)a.z}; }
+template <typename T> inline V3T<T> operator+(V3T<T> a, V3T<T> b) { return V3T<T>{a.x + b.x, a.y + b.y, a.z + b.z}; }
+template <typename T> inline V3T<T> operator-(V3T<T> a, V3T<T> b) { return V3T<T>{a.x - b.x, a.y - b.y, a.z - b.z}; }
+template <typename T> inline V3T<T> operator-(V3T<T> a) { return V3T<T>{-a.x, -a.y, -a.z}; }
+template <typename T, typename S> inline V3T<T> operator*(V3T<T> a, S s) { return V3T<T>{a.x * (T)s, a.y * (T)s, a.z * (T)s}; }
+template <typename T, typename S> inline V3T<T> operator*(S s, V3T<T> a) { return V3T<T>{(T)s * a.x, (T)s * a.y, (T)s * a.z}; }
+template <typename T, typename S> inline V3T<T> operator/(V3T<T> a, S s) { return V3T<T>{a.x / (T)s, a.y / (T)s, a.z / (T)s}; }
+template <typename T> inline T dot(V3T<T> a, V3T<T> b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+template <typename T> inline V3T<T> cross(V3T<T> a, V3T<T> b) {
+    return V3T<T>{a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
+}
+template <typename T> inline T len(V3T<T> a) { return std::sqrt(dot(a, a)); }
 
 struct Hit { float t; uint32_t idx; };
 
@@ -132,9 +140,10 @@ inline void quat_rows(const float *q, V3 R[3]) {
 }
 
 // auxiliary.h:433-477 (no Jacobian of the normalisation)
-inline void quat_rows_vjp(const float *q, const V3 g[3], float out[4]) {
-    float s = 1.0f / std::sqrt(q[3] * q[3] + q[0] * q[0] + q[1] * q[1] + q[2] * q[2]);
-    float w = q[0] * s, x = q[1] * s, y = q[2] * s, z = q[3] * s;
+template <typename T> inline void quat_rows_vjp(const float *qf, const V3T<T> g[3], T out[4]) {
+    const T q[4] = {(T)qf[0], (T)qf[1], (T)qf[2], (T)qf[3]};
+    T s = (T)1.0f / std::sqrt(q[3] * q[3] + q[0] * q[0] + q[1] * q[1] + q[2] * q[2]);
+    T w = q[0] * s, x = q[1] * s, y = q[2] * s, z = q[3] * s;
     out[0] = 2.f * (x * (g[1].z - g[2].y) + y * (g[2].x - g[0].z) + z * (g[0].y - g[1].x));
     out[1] = 2.f * (-2.f * x * (g[1].y + g[2].z) + y * (g[0].y + g[1].x) + z * (g[0].z + g[2].x) + w * (g[1].z - g[2].y));
     out[2] = 2.f * (x * (g[0].y + g[1].x) - 2.f * y * (g[0].x + g[2].z) + z * (g[1].z + g[2].y) + w * (g[2].x - g[0].z));
@@ -169,13 +178,15 @@ inline V3 sh_color(int deg, const float *sh, V3 dir, float clamped[3]) {
 }
 
 // backward.cu:68-166.  g_sh receives (deg+1)^2 float3; g_dir is ASSIGNED (backward.cu:165).
-inline void sh_color_backward(int deg, const float *sh, V3 dir, const float clamped[3], const float g_col[3],
-                              V3 *g_sh, V3 &g_dir) {
-    auto S = [&](int j) { return ld3(sh + 3 * j); };
-    V3 g = v3(g_col[0] * (clamped[0] != 0.f ? 0.f : 1.f), g_col[1] * (clamped[1] != 0.f ? 0.f : 1.f),
-              g_col[2] * (clamped[2] != 0.f ? 0.f : 1.f));
-    V3 dx = v3(0, 0, 0), dy = v3(0, 0, 0), dz = v3(0, 0, 0);
-    float x = dir.x, y = dir.y, z = dir.z;
+template <typename T>
+inline void sh_color_backward(int deg, const float *sh, V3 dirf, const float clamped[3], const T g_col[3],
+                              V3T<T> *g_sh, V3T<T> &g_dir) {
+    using W3 = V3T<T>;
+    auto S = [&](int j) { return cast3<T>(ld3(sh + 3 * j)); };
+    W3 g = v3t<T>(g_col[0] * (clamped[0] != 0.f ? 0.f : 1.f), g_col[1] * (clamped[1] != 0.f ? 0.f : 1.f),
+                  g_col[2] * (clamped[2] != 0.f ? 0.f : 1.f));
+    W3 dx = v3t<T>(0, 0, 0), dy = v3t<T>(0, 0, 0), dz = v3t<T>(0, 0, 0);
+    T x = dirf.x, y = dirf.y, z = dirf.z;
     g_sh[0] = C0 * g;
     if (deg > 0) {
         g_sh[1] = (-C1 * y) * g;
@@ -185,7 +196,7 @@ inline void sh_color_backward(int deg, const float *sh, V3 dir, const float clam
         dy = -C1 * S(1);
         dz = C1 * S(2);
         if (deg > 1) {
-            float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+            T xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
             g_sh[4] = (C2[0] * xy) * g;
             g_sh[5] = (C2[1] * yz) * g;
             g_sh[6] = (C2[2] * (2.f * zz - xx - yy)) * g;
@@ -214,7 +225,7 @@ inline void sh_color_backward(int deg, const float *sh, V3 dir, const float clam
             }
         }
     }
-    g_dir = v3(dot(dx, g), dot(dy, g), dot(dz, g));
+    g_dir = v3t<T>(dot(dx, g), dot(dy, g), dot(dz, g));
 }
 
 // ---- world -> splat; forward.cu:63-90 ------------------------------------------------------------
@@ -455,6 +466,10 @@ void k_nearest(const Scene &sc, V3 o, V3 d, Hit buf[kChunk], uint32_t &cnt) {
 // ---- per-surfel accumulators (double, rounded once at the end) ----------------------------------------
 struct Accum {
     std::vector<double> w, means, grads, shs, colors, others, opac, scales, rots;
+    // optional (backward with grad_f64 and noise outputs): summed first-order sensitivity of the geometric
+    // gradients to fp32 rounding of the plane-hit chain
+    bool noise = false;
+    std::vector<double> n_means, n_grads, n_scales, n_rots;
 };
 inline void aadd(std::vector<double> &v, size_t i, double x) {
     double *d = v.data();
@@ -589,31 +604,42 @@ void path_forward(const Scene &sc, V3 ray_o, V3 ray_d, float *out_rgb, float &ou
 }
 
 // backward.cu:201-287
-struct GeoGrad { float scale[2], rot[4]; V3 mean; };
-void splat_uv_backward(const float *mean, const float *scale, const float *rot, V3 xyz, const Splat &s,
-                       float normal_sign, V3 ray_o, V3 ray_d, float dpt, V3 v1, V3 v2, V3 v3_, V3 h1, V3 h2, V3 h3,
-                       float G, float pclamp, V3 g_N, float g_D, float g_G, V3 &g_ray_o, V3 &g_ray_d, GeoGrad &out) {
-    V3 pm = ld3(mean);
-    float sx = scale[0], sy = scale[1];
-    float gu = g_G * pclamp * -G * s.u, gv = g_G * pclamp * -G * s.v;
-    V3 gR[3];
+template <typename T> struct GeoGrad { T scale[2], rot[4]; V3T<T> mean; };
+template <typename T>
+void splat_uv_backward(const float *mean, const float *scale, const float *rot, V3 xyzf, const Splat &sf,
+                       float normal_sign, V3 ray_of, V3 ray_df, float dptf, V3 v1f, V3 v2f, V3 v3f, V3 h1, V3 h2, V3 h3,
+                       float Gf, float pclamp, V3T<T> g_N, T g_D, T g_G, V3T<T> &g_ray_o, V3T<T> &g_ray_d,
+                       GeoGrad<T> &out, int perturb = 0) {
+    using W3 = V3T<T>;
+    const W3 pm = cast3<T>(ld3(mean)), xyz = cast3<T>(xyzf), ray_o = cast3<T>(ray_of), ray_d = cast3<T>(ray_df);
+    const W3 v1 = cast3<T>(v1f), v2 = cast3<T>(v2f), v3_ = cast3<T>(v3f);
+    const W3 R0 = cast3<T>(sf.R[0]), R1 = cast3<T>(sf.R[1]);
+    const T sx = scale[0], sy = scale[1], G = Gf, su_ = sf.u, sv_ = sf.v, dpt = dptf;
+    T gu = g_G * pclamp * -G * su_, gv = g_G * pclamp * -G * sv_;
+    W3 gR[3];
     gR[0] = gu * (xyz - pm) / sx;
     gR[1] = gv * (xyz - pm) / sy;
     gR[2] = g_N * normal_sign;
-    out.scale[0] = g_G * pclamp * (G * s.u * s.u / sx);
-    out.scale[1] = g_G * pclamp * (G * s.v * s.v / sy);
-    V3 dG_dmean = G * (s.R[0] * s.u / sx + s.R[1] * s.v / sy);
+    out.scale[0] = g_G * pclamp * (G * su_ * su_ / sx);
+    out.scale[1] = g_G * pclamp * (G * sv_ * sv_ / sy);
+    W3 dG_dmean = G * (R0 * su_ / sx + R1 * sv_ / sy);
     out.mean = g_G * pclamp * dG_dmean;
-    V3 g_xyz = v3(gu / sx * s.R[0].x + gv / sy * s.R[1].x, gu / sx * s.R[0].y + gv / sy * s.R[1].y,
-                  gu / sx * s.R[0].z + gv / sy * s.R[1].z);
-    float g_d = g_D + dot(g_xyz, ray_d);
-    V3 n = cross(v2 - v1, v3_ - v1);
-    V3 c = v1 - ray_o;
-    float pp = dot(n, c), q = dot(n, ray_d);
-    V3 g_n = (c - pp / q * ray_d) / q;
-    V3 g_v1 = g_d * cross(v2 - v3_, g_n) + g_d * n / q;
-    V3 g_v2 = g_d * cross(v3_ - v1, g_n);
-    V3 g_v3 = g_d * cross(v1 - v2, g_n);
+    W3 g_xyz = v3t<T>(gu / sx * R0.x + gv / sy * R1.x, gu / sx * R0.y + gv / sy * R1.y, gu / sx * R0.z + gv / sy * R1.z);
+    T g_d = g_D + dot(g_xyz, ray_d);
+    W3 n = cross(v2 - v1, v3_ - v1);
+    W3 c = v1 - ray_o;
+    // `perturb` (sensitivity estimate only): move one rounded intermediate of the plane-hit chain by one unit of
+    // fp32 rounding of the operands it was computed from
+    const T ulp = (T)1.1920929e-7f;
+    if (perturb == 3) c = c + v3t<T>(ulp * (std::abs(v1.x) + std::abs(ray_o.x)), ulp * (std::abs(v1.y) + std::abs(ray_o.y)),
+                                     ulp * (std::abs(v1.z) + std::abs(ray_o.z)));
+    T pp = dot(n, c), q = dot(n, ray_d);
+    if (perturb == 1) pp += ulp * (std::abs(n.x * c.x) + std::abs(n.y * c.y) + std::abs(n.z * c.z));
+    if (perturb == 2) q += ulp * (std::abs(n.x * ray_d.x) + std::abs(n.y * ray_d.y) + std::abs(n.z * ray_d.z));
+    W3 g_n = (c - pp / q * ray_d) / q;
+    W3 g_v1 = g_d * cross(v2 - v3_, g_n) + g_d * n / q;
+    W3 g_v2 = g_d * cross(v3_ - v1, g_n);
+    W3 g_v3 = g_d * cross(v1 - v2, g_n);
     g_ray_o = g_ray_o + (g_xyz + g_d * -n / q);
     g_ray_d = g_ray_d + (g_xyz * dpt + g_d * -pp / (q * q) * n);
     gR[0].x += sx * (h1.x * g_v1.x + h2.x * g_v2.x + h3.x * g_v3.x);
@@ -622,22 +648,25 @@ void splat_uv_backward(const float *mean, const float *scale, const float *rot, 
     gR[1].x += sy * (h1.y * g_v1.x + h2.y * g_v2.x + h3.y * g_v3.x);
     gR[1].y += sy * (h1.y * g_v1.y + h2.y * g_v2.y + h3.y * g_v3.y);
     gR[1].z += sy * (h1.y * g_v1.z + h2.y * g_v2.z + h3.y * g_v3.z);
-    quat_rows_vjp(rot, gR, out.rot);
-    out.scale[0] += dot(s.R[0], h1.x * g_v1 + h2.x * g_v2 + h3.x * g_v3);
-    out.scale[1] += dot(s.R[1], h1.y * g_v1 + h2.y * g_v2 + h3.y * g_v3);
+    quat_rows_vjp<T>(rot, gR, out.rot);
+    out.scale[0] += dot(R0, h1.x * g_v1 + h2.x * g_v2 + h3.x * g_v3);
+    out.scale[1] += dot(R1, h1.y * g_v1 + h2.y * g_v2 + h3.y * g_v3);
     out.mean = out.mean + (g_v1 + g_v2 + g_v3);
 }
 
+template <typename T>
 struct BounceIn {  // saved results of this bounce and its upstream gradients
     float rgb[3], dpt, acc, aux[kMaxAux];
     V3 norm;
-    float g_rgb[3], g_dpt, g_acc, g_aux[kMaxAux];
-    V3 g_norm;
+    T g_rgb[3], g_dpt, g_acc, g_aux[kMaxAux];
+    V3T<T> g_norm;
 };
 
 // backward.cu:332-655
-void bounce_backward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float T_threshold, const BounceIn &in,
-                     V3 &g_ray_o, V3 &g_ray_d, Accum &acc) {
+template <typename T>
+void bounce_backward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float T_threshold, const BounceIn<T> &in,
+                     V3T<T> &g_ray_o, V3T<T> &g_ray_d, Accum &acc, V3T<T> *n_ray_o = nullptr,
+                     V3T<T> *n_ray_d = nullptr) {
     const OracleParams *p = sc.p;
     Hit buf[kChunk];
     for (int i = 0; i < kChunk; ++i) buf[i] = Hit{kInfDepth, 0u};
@@ -701,35 +730,37 @@ void bounce_backward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float
             D += w * dpt;
             N = v3(N.x + w * normal.x, N.y + w * normal.y, N.z + w * normal.z);
 
-            // gradient of this hit (backward.cu:528-640)
-            float g_alpha = 0.0f;
-            const float num = 1.0f - alpha;
-            float g_color[3];
+            // gradient of this hit (backward.cu:528-640); T = float is the restatement, T = double the same
+            // formulas on the same fp32 inputs and decisions
+            T g_alpha = 0.0f;
+            const T num = (T)1.0f - (T)alpha;
+            const T Tp = T_prev, wT = w;
+            T g_color[3];
             for (int ch = 0; ch < 3; ++ch) {
-                g_color[ch] = in.g_rgb[ch] * w;
-                aadd(acc.colors, ch + 3 * (size_t)g, (double)(in.g_rgb[ch] * w));
-                g_alpha += in.g_rgb[ch] * (T_prev * c[ch] - (in.rgb[ch] - C[ch]) / num);
-                g_alpha += in.g_rgb[ch] * p->background[ch] * (-T_final / num);
+                g_color[ch] = in.g_rgb[ch] * wT;
+                aadd(acc.colors, ch + 3 * (size_t)g, (double)(in.g_rgb[ch] * wT));
+                g_alpha += in.g_rgb[ch] * (Tp * (T)c[ch] - ((T)in.rgb[ch] - (T)C[ch]) / num);
+                g_alpha += in.g_rgb[ch] * (T)p->background[ch] * (-(T)T_final / num);
             }
             if (p->others_precomp != nullptr) {
                 for (int ch = 0; ch < p->aux; ++ch) {
-                    float o = p->others_precomp[ch + (size_t)p->aux * g];
-                    aadd(acc.others, ch + (size_t)p->aux * g, (double)(in.g_aux[ch] * w));
-                    g_alpha += in.g_aux[ch] * (T_prev * o - (in.aux[ch] - O[ch]) / num);
+                    T o = p->others_precomp[ch + (size_t)p->aux * g];
+                    aadd(acc.others, ch + (size_t)p->aux * g, (double)(in.g_aux[ch] * wT));
+                    g_alpha += in.g_aux[ch] * (Tp * o - ((T)in.aux[ch] - (T)O[ch]) / num);
                 }
             }
-            float g_D = in.g_dpt * w;
-            g_alpha += in.g_dpt * (T_prev * dpt - (in.dpt - D) / num);
-            V3 g_N = in.g_norm * w;
+            T g_D = in.g_dpt * wT;
+            g_alpha += in.g_dpt * (Tp * (T)dpt - ((T)in.dpt - (T)D) / num);
+            V3T<T> g_N = in.g_norm * wT;
             {
-                V3 tn = T_prev * normal - (in.norm - N) / num;
+                V3T<T> tn = Tp * cast3<T>(normal) - (cast3<T>(in.norm) - cast3<T>(N)) / num;
                 g_alpha += in.g_norm.x * tn.x + in.g_norm.y * tn.y + in.g_norm.z * tn.z;
             }
-            g_alpha += in.g_acc * (T_prev * 1.f - (in.acc - W) / num);
+            g_alpha += in.g_acc * (Tp * 1.f - ((T)in.acc - (T)W) / num);
             const float opac = p->opacities[g];
-            const float g_G = g_alpha * opac;
+            const T g_G = g_alpha * (T)opac;
             float pclamp = (opac * G) > 0.99f ? 0.0f : 1.0f;
-            aadd(acc.opac, (size_t)g, (double)(g_alpha * G * pclamp));
+            aadd(acc.opac, (size_t)g, (double)(g_alpha * (T)G * pclamp));
             const float *V = p->vertices + (size_t)g * 12;
             V3 v1, v2, v3_, h1, h2, h3;
             if (pidx % 2 == 0) {
@@ -739,21 +770,46 @@ void bounce_backward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float
                 v1 = ld3(V + 3); v2 = ld3(V + 6); v3_ = ld3(V + 9);
                 h1 = v3(-1.f, -1.f, 1.f) * cutoff; h2 = v3(1.f, 1.f, 1.f) * cutoff; h3 = v3(1.f, -1.f, 1.f) * cutoff;
             }
-            GeoGrad gg;
-            splat_uv_backward(mean, scale, rot, xyz, s, normal_sign, ray_o, ray_d, dpt, v1, v2, v3_, h1, h2, h3, G,
-                              pclamp, g_N, g_D, g_G, g_ray_o, g_ray_d, gg);
+            GeoGrad<T> gg;
+            splat_uv_backward<T>(mean, scale, rot, xyz, s, normal_sign, ray_o, ray_d, dpt, v1, v2, v3_, h1, h2, h3, G,
+                                 pclamp, g_N, g_D, g_G, g_ray_o, g_ray_d, gg);
+            if (acc.noise) {
+                GeoGrad<T> gb;
+                V3T<T> bo = v3t<T>(0, 0, 0), bd = v3t<T>(0, 0, 0);
+                splat_uv_backward<T>(mean, scale, rot, xyz, s, normal_sign, ray_o, ray_d, dpt, v1, v2, v3_, h1, h2, h3, G,
+                                     pclamp, g_N, g_D, g_G, bo, bd, gb, 0);
+                for (int pert = 1; pert <= 3; ++pert) {
+                    GeoGrad<T> gq;
+                    V3T<T> qo = v3t<T>(0, 0, 0), qd = v3t<T>(0, 0, 0);
+                    splat_uv_backward<T>(mean, scale, rot, xyz, s, normal_sign, ray_o, ray_d, dpt, v1, v2, v3_, h1, h2, h3,
+                                         G, pclamp, g_N, g_D, g_G, qo, qd, gq, pert);
+                    for (int k = 0; k < 2; ++k) aadd(acc.n_scales, 2 * (size_t)g + k, std::abs((double)(gq.scale[k] - gb.scale[k])));
+                    for (int k = 0; k < 4; ++k) aadd(acc.n_rots, 4 * (size_t)g + k, std::abs((double)(gq.rot[k] - gb.rot[k])));
+                    const double dm[3] = {std::abs((double)(gq.mean.x - gb.mean.x)), std::abs((double)(gq.mean.y - gb.mean.y)),
+                                          std::abs((double)(gq.mean.z - gb.mean.z))};
+                    for (int k = 0; k < 3; ++k) {
+                        aadd(acc.n_means, 3 * (size_t)g + k, dm[k]);
+                        aadd(acc.n_grads, 3 * (size_t)g + k, dm[k] * 0.5 * (double)dpt);
+                    }
+                    if (n_ray_o && n_ray_d) {
+                        *n_ray_o = *n_ray_o + v3t<T>(std::abs(qo.x - bo.x), std::abs(qo.y - bo.y), std::abs(qo.z - bo.z));
+                        *n_ray_d = *n_ray_d + v3t<T>(std::abs(qd.x - bd.x), std::abs(qd.y - bd.y), std::abs(qd.z - bd.z));
+                    }
+                }
+            }
             aadd(acc.scales, 2 * (size_t)g + 0, gg.scale[0]);
             aadd(acc.scales, 2 * (size_t)g + 1, gg.scale[1]);
             for (int k = 0; k < 4; ++k) aadd(acc.rots, 4 * (size_t)g + k, gg.rot[k]);
             aadd(acc.means, 3 * (size_t)g + 0, gg.mean.x);
             aadd(acc.means, 3 * (size_t)g + 1, gg.mean.y);
             aadd(acc.means, 3 * (size_t)g + 2, gg.mean.z);
-            aadd(acc.grads, 3 * (size_t)g + 0, gg.mean.x * 0.5f * dpt);
-            aadd(acc.grads, 3 * (size_t)g + 1, gg.mean.y * 0.5f * dpt);
-            aadd(acc.grads, 3 * (size_t)g + 2, gg.mean.z * 0.5f * dpt);
+            aadd(acc.grads, 3 * (size_t)g + 0, gg.mean.x * 0.5f * (T)dpt);
+            aadd(acc.grads, 3 * (size_t)g + 1, gg.mean.y * 0.5f * (T)dpt);
+            aadd(acc.grads, 3 * (size_t)g + 2, gg.mean.z * 0.5f * (T)dpt);
             if (p->colors_precomp == nullptr) {
-                V3 g_sh[16];
-                sh_color_backward(p->D, p->shs + (size_t)g * p->M * 3, ray_d, clamped, g_color, g_sh, g_ray_d);
+                V3T<T> g_sh[16];
+                sh_color_backward<T>(p->D, p->shs + (size_t)g * p->M * 3, ray_d, clamped, g_color, g_sh, g_ray_d);
+                if (n_ray_d) *n_ray_d = v3t<T>(0, 0, 0);   // the direction gradient was just replaced (backward.cu:165)
                 for (int j = 0; j < (p->D + 1) * (p->D + 1); ++j) {
                     aadd(acc.shs, ((size_t)g * p->M + j) * 3 + 0, g_sh[j].x);
                     aadd(acc.shs, ((size_t)g * p->M + j) * 3 + 1, g_sh[j].y);
@@ -772,47 +828,49 @@ void bounce_backward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float
 }
 
 // auxiliary.h:111-121
-inline V3 dnormvdv(V3 v, V3 dv) {
-    float sum2 = v.x * v.x + v.y * v.y + v.z * v.z;
-    float inv = 1.0f / std::sqrt(sum2 * sum2 * sum2);
-    return v3(((+sum2 - v.x * v.x) * dv.x - v.y * v.x * dv.y - v.z * v.x * dv.z) * inv,
-              (-v.x * v.y * dv.x + (sum2 - v.y * v.y) * dv.y - v.z * v.y * dv.z) * inv,
-              (-v.x * v.z * dv.x - v.y * v.z * dv.y + (sum2 - v.z * v.z) * dv.z) * inv);
+template <typename T> inline V3T<T> dnormvdv(V3T<T> v, V3T<T> dv) {
+    T sum2 = v.x * v.x + v.y * v.y + v.z * v.z;
+    T inv = (T)1.0f / std::sqrt(sum2 * sum2 * sum2);
+    return v3t<T>(((+sum2 - v.x * v.x) * dv.x - v.y * v.x * dv.y - v.z * v.x * dv.z) * inv,
+                  (-v.x * v.y * dv.x + (sum2 - v.y * v.y) * dv.y - v.z * v.y * dv.z) * inv,
+                  (-v.x * v.z * dv.x - v.y * v.z * dv.y + (sum2 - v.z * v.z) * dv.z) * inv);
 }
 // auxiliary.h:234-252
-inline V3 ddotndndn(V3 n, V3 d, V3 g) {
-    float nd = dot(n, d);
-    return v3(g.x * (nd + d.x * n.x) + g.y * d.x * n.y + g.z * d.x * n.z,
-              g.x * d.y * n.x + g.y * (nd + d.y * n.y) + g.z * d.y * n.z,
-              g.x * d.z * n.x + g.y * d.z * n.y + g.z * (nd + d.z * n.z));
+template <typename T> inline V3T<T> ddotndndn(V3T<T> n, V3T<T> d, V3T<T> g) {
+    T nd = dot(n, d);
+    return v3t<T>(g.x * (nd + d.x * n.x) + g.y * d.x * n.y + g.z * d.x * n.z,
+                  g.x * d.y * n.x + g.y * (nd + d.y * n.y) + g.z * d.y * n.z,
+                  g.x * d.z * n.x + g.y * d.z * n.y + g.z * (nd + d.z * n.z));
 }
-inline V3 ddotndndd(V3 n, V3 /*d*/, V3 g) {
-    return v3(g.x * n.x * n.x + g.y * n.x * n.y + g.z * n.x * n.z, g.x * n.y * n.x + g.y * n.y * n.y + g.z * n.y * n.z,
-              g.x * n.z * n.x + g.y * n.z * n.y + g.z * n.z * n.z);
+template <typename T> inline V3T<T> ddotndndd(V3T<T> n, V3T<T> /*d*/, V3T<T> g) {
+    return v3t<T>(g.x * n.x * n.x + g.y * n.x * n.y + g.z * n.x * n.z, g.x * n.y * n.x + g.y * n.y * n.y + g.z * n.y * n.z,
+                  g.x * n.z * n.x + g.y * n.z * n.y + g.z * n.z * n.z);
 }
 
 // backward.cu:658-853
+template <typename T>
 void path_backward(const Scene &sc, const float *out_rgb, const float *mid, const float *g_out_rgb, float g_out_dpt,
-                   float g_out_acc, V3 g_out_norm, const float *g_out_aux, V3 &g_ray_o, V3 &g_ray_d, Accum &acc) {
+                   float g_out_acc, V3 g_out_norm, const float *g_out_aux, V3T<T> &g_ray_o, V3T<T> &g_ray_d, Accum &acc,
+                   V3T<T> *n_ray_o = nullptr, V3T<T> *n_ray_d = nullptr) {
     const OracleParams *p = sc.p;
     const int MID = mid_channels(p), AUXO = 11, RGBO = 11 + p->aux, mtd = p->max_trace_depth;
-    float C_prev[3], c_prev[3] = {0, 0, 0};
+    T C_prev[3], c_prev[3] = {0, 0, 0};
     for (int ch = 0; ch < 3; ++ch) C_prev[ch] = out_rgb[ch];
-    float s_prod = 1.0f;
+    T s_prod = 1.0f;
     for (int i = 0; i < mtd; ++i) {
         for (int ch = 0; ch < 3; ++ch) {
-            float c_curr = mid[ch + RGBO + i * MID];
+            T c_curr = mid[ch + RGBO + i * MID];
             C_prev[ch] = C_prev[ch] + s_prod * (c_prev[ch] - c_curr);
             c_prev[ch] = c_curr;
         }
-        s_prod *= mid[AUXO + i * MID];
+        s_prod *= (T)mid[AUXO + i * MID];
     }
     for (int i = mtd; i >= 0; --i) {
         const float *m = mid + (size_t)i * MID;
         V3 ot = ld3(m + 0), dt = ld3(m + 3);
         float s_prev = (i > 0) ? mid[AUXO + (i - 1) * MID] : 1.0f;
         if (len(dt) == 0.0f || s_prev <= p->specular_threshold) continue;
-        BounceIn in;
+        BounceIn<T> in;
         for (int ch = 0; ch < 3; ++ch) in.rgb[ch] = m[RGBO + ch];
         in.dpt = m[6];
         in.acc = m[7];
@@ -820,33 +878,34 @@ void path_backward(const Scene &sc, const float *out_rgb, const float *mid, cons
         for (int ch = 0; ch < kMaxAux; ++ch) in.aux[ch] = (ch < p->aux) ? m[AUXO + ch] : 0.f;
         in.g_dpt = 0.f;
         in.g_acc = 0.f;
-        in.g_norm = v3(0, 0, 0);
+        in.g_norm = v3t<T>(0, 0, 0);
         for (int ch = 0; ch < kMaxAux; ++ch) in.g_aux[ch] = 0.f;
         float f_this = (i == mtd) ? 1.0f : 1 - in.aux[0];
-        for (int ch = 0; ch < 3; ++ch) in.g_rgb[ch] = g_out_rgb[ch] * f_this * s_prod;
-        s_prod /= s_prev;
+        for (int ch = 0; ch < 3; ++ch) in.g_rgb[ch] = (T)g_out_rgb[ch] * (T)f_this * s_prod;
+        s_prod /= (T)s_prev;
         if (i != mtd) {
             for (int ch = 0; ch < 3; ++ch) {
-                in.g_aux[0] += g_out_rgb[ch] * (C_prev[ch] / in.aux[0]);
+                in.g_aux[0] += (T)g_out_rgb[ch] * (C_prev[ch] / (T)in.aux[0]);
                 c_prev[ch] = (i > 0) ? mid[ch + RGBO + (i - 1) * MID] : 0.0f;
-                C_prev[ch] = C_prev[ch] - s_prod * (c_prev[ch] - in.rgb[ch]);
+                C_prev[ch] = C_prev[ch] - s_prod * (c_prev[ch] - (T)in.rgb[ch]);
             }
             if (len(in.norm) != 0) {
-                g_ray_d = g_ray_d + g_ray_o * (float)kStepEps;
-                V3 n = in.norm / len(in.norm);
-                in.g_dpt += g_ray_o.x * dt.x + g_ray_o.y * dt.y + g_ray_o.z * dt.z;
-                in.g_norm = in.g_norm + dnormvdv(in.norm, ddotndndn(n, dt, g_ray_d * -2.0f));
-                g_ray_d = g_ray_o * in.dpt + g_ray_d + ddotndndd(n, dt, g_ray_d * -2.0f);
+                const V3T<T> normT = cast3<T>(in.norm), dtT = cast3<T>(dt);
+                g_ray_d = g_ray_d + g_ray_o * (T)(float)kStepEps;
+                V3T<T> n = normT / len(normT);
+                in.g_dpt += g_ray_o.x * dtT.x + g_ray_o.y * dtT.y + g_ray_o.z * dtT.z;
+                in.g_norm = in.g_norm + dnormvdv<T>(normT, ddotndndn<T>(n, dtT, g_ray_d * -2.0f));
+                g_ray_d = g_ray_o * (T)in.dpt + g_ray_d + ddotndndd<T>(n, dtT, g_ray_d * -2.0f);
             }
         }
         if (i == 0) {
             in.g_dpt += g_out_dpt;
             in.g_acc += g_out_acc;
-            in.g_norm = in.g_norm + g_out_norm;
+            in.g_norm = in.g_norm + cast3<T>(g_out_norm);
             for (int ch = 0; ch < p->aux; ++ch) in.g_aux[ch] += g_out_aux[ch];
         }
         float min_depth = (i == 0 && p->start_from_first) ? kNear : (i == 0 && !p->start_from_first) ? 0.0f : kStartOffset;
-        bounce_backward(sc, ot, dt, min_depth, kTmin, in, g_ray_o, g_ray_d, acc);
+        bounce_backward<T>(sc, ot, dt, min_depth, kTmin, in, g_ray_o, g_ray_d, acc, n_ray_o, n_ray_d);
     }
 }
 
@@ -900,6 +959,14 @@ int oracle_ray_quad(const float *o, const float *d, const float *A, const float 
     *t = tt;
     *tri = k;
     return hit ? 1 : 0;
+}
+
+void oracle_reflection_vjp(int which, const float *a, const float *b, const float *g, float *out) {
+    V3 r = v3(0, 0, 0);
+    if (which == 0) r = dnormvdv<float>(ld3(a), ld3(g));                 // a = v
+    else if (which == 1) r = ddotndndn<float>(ld3(a), ld3(b), ld3(g));   // a = n, b = d
+    else if (which == 2) r = ddotndndd<float>(ld3(a), ld3(b), ld3(g));
+    out[0] = r.x; out[1] = r.y; out[2] = r.z;
 }
 
 int oracle_k_nearest(const OracleParams *p, const float *o, const float *d, float *t16, uint32_t *idx16) {
@@ -968,16 +1035,38 @@ int oracle_trace_backward(const OracleParams *p) {
     acc.opac.assign(P, 0.0);
     acc.scales.assign(P * 2, 0.0);
     acc.rots.assign(P * 4, 0.0);
+    acc.noise = p->grad_f64 && p->noise_ray_o && p->noise_ray_d && p->noise_means3D && p->noise_grads3D &&
+                p->noise_scales && p->noise_rotations;
+    if (acc.noise) {
+        acc.n_means.assign(P * 3, 0.0);
+        acc.n_grads.assign(P * 3, 0.0);
+        acc.n_scales.assign(P * 2, 0.0);
+        acc.n_rots.assign(P * 4, 0.0);
+    }
     const auto t_start = std::chrono::steady_clock::now();
 #pragma omp parallel for schedule(dynamic, 64)
     for (long r = 0; r < R; ++r) {
         float g_aux[kMaxAux] = {0};
         for (int ch = 0; ch < p->aux; ++ch) g_aux[ch] = p->dL_daux[(size_t)p->aux * r + ch];
-        V3 g_o = v3(0, 0, 0), g_d = v3(0, 0, 0);
-        path_backward(sc, p->out_rgb + 3 * r, p->mid_val + (size_t)slots * MID * r, p->dL_drgb + 3 * r, p->dL_ddpt[r],
-                      p->dL_dacc[r], ld3(p->dL_dnorm + 3 * r), g_aux, g_o, g_d, acc);
-        p->dL_dray_o[3 * r + 0] = g_o.x; p->dL_dray_o[3 * r + 1] = g_o.y; p->dL_dray_o[3 * r + 2] = g_o.z;
-        p->dL_dray_d[3 * r + 0] = g_d.x; p->dL_dray_d[3 * r + 1] = g_d.y; p->dL_dray_d[3 * r + 2] = g_d.z;
+        const float *rgb = p->out_rgb + 3 * r, *mid = p->mid_val + (size_t)slots * MID * r, *g_rgb = p->dL_drgb + 3 * r;
+        if (p->grad_f64) {
+            V3T<double> g_o = v3t<double>(0, 0, 0), g_d = v3t<double>(0, 0, 0);
+            V3T<double> n_o = v3t<double>(0, 0, 0), n_d = v3t<double>(0, 0, 0);
+            path_backward<double>(sc, rgb, mid, g_rgb, p->dL_ddpt[r], p->dL_dacc[r], ld3(p->dL_dnorm + 3 * r), g_aux, g_o,
+                                  g_d, acc, &n_o, &n_d);
+            if (acc.noise) {
+                p->noise_ray_o[3 * r + 0] = (float)n_o.x; p->noise_ray_o[3 * r + 1] = (float)n_o.y; p->noise_ray_o[3 * r + 2] = (float)n_o.z;
+                p->noise_ray_d[3 * r + 0] = (float)n_d.x; p->noise_ray_d[3 * r + 1] = (float)n_d.y; p->noise_ray_d[3 * r + 2] = (float)n_d.z;
+            }
+            p->dL_dray_o[3 * r + 0] = (float)g_o.x; p->dL_dray_o[3 * r + 1] = (float)g_o.y; p->dL_dray_o[3 * r + 2] = (float)g_o.z;
+            p->dL_dray_d[3 * r + 0] = (float)g_d.x; p->dL_dray_d[3 * r + 1] = (float)g_d.y; p->dL_dray_d[3 * r + 2] = (float)g_d.z;
+        } else {
+            V3 g_o = v3(0, 0, 0), g_d = v3(0, 0, 0);
+            path_backward<float>(sc, rgb, mid, g_rgb, p->dL_ddpt[r], p->dL_dacc[r], ld3(p->dL_dnorm + 3 * r), g_aux, g_o,
+                                 g_d, acc);
+            p->dL_dray_o[3 * r + 0] = g_o.x; p->dL_dray_o[3 * r + 1] = g_o.y; p->dL_dray_o[3 * r + 2] = g_o.z;
+            p->dL_dray_d[3 * r + 0] = g_d.x; p->dL_dray_d[3 * r + 1] = g_d.y; p->dL_dray_d[3 * r + 2] = g_d.z;
+        }
     }
     if (p->trace_seconds)
         *p->trace_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_start).count();
@@ -989,6 +1078,12 @@ int oracle_trace_backward(const OracleParams *p) {
     flush(acc.opac, p->dL_dopacities);
     flush(acc.scales, p->dL_dscales);
     flush(acc.rots, p->dL_drotations);
+    if (acc.noise) {
+        flush(acc.n_means, p->noise_means3D);
+        flush(acc.n_grads, p->noise_grads3D);
+        flush(acc.n_scales, p->noise_scales);
+        flush(acc.n_rots, p->noise_rotations);
+    }
     return 0;
 }
 

@@ -10,19 +10,19 @@
  * of the reference tree) is DEFINED here, see surfel_oracle.cpp: parity of
  * that part against OptiX itself is unpinned.
  *
- * Parity unpinned (transcribed from the cited lines and reviewed, but checked
- * by no independent test, because the reference deviates from the true
- * gradient there and nothing but the reference itself says how):
- *   - bounce_backward(): the flow of dL/dacc (the reference never accumulates
- *     the weight sum W, backward.cu:568);
- *   - path_backward(): the part of a bounce's gradient that reaches the
- *     previous bounce through the reflected ray's origin and direction
- *     (backward.cu:700-790).
+ * Parity unpinned: only the hit enumeration named above (the set of hits, the value
+ * of t and the order of exactly tied depths as NVIDIA's OptiX would report them).
  * Everything else is pinned by tests/test_oracle_*.py: scalar functions against
  * numpy/scipy, the ray/quad test against float64 Moeller-Trumbore, hit ordering
- * against brute force, compositing against closed forms, gradients (depth 0
- * and the bounce weighting at depth 1) against torch autograd of an
- * independent float64 forward.
+ * against brute force, compositing against closed forms, and every gradient
+ * against torch autograd of an independent float64 forward: depth 0, the flow of
+ * dL/dacc (the reference never accumulates the weight sum W, backward.cu:568:
+ * differentiated as the surrogate it is the exact gradient of), the helpers of
+ * the reflection chain rule as Jacobians, and the whole multi-bounce chain with
+ * the reflected rays left free (backward.cu:700-790; depth 1 and depth 2).
+ * The kernel's text of the small formulas (exp, quaternion frame, SH
+ * polynomials, ray/quad test) is the same as the text here, not an independent
+ * derivation; those four are the ones pinned against numpy/scipy for that reason.
  */
 #ifndef SURFEL_ORACLE_H
 #define SURFEL_ORACLE_H
@@ -52,6 +52,10 @@ typedef struct OracleParams {
     int32_t hit_mode;      /* ORACLE_HITS_* */
     int32_t literal_stale; /* 1: keep the reference's stale slot on a repeated surfel (forward.cu:207-208) */
     int32_t n_threads;     /* OpenMP threads, 0 = default */
+    int32_t grad_f64;      /* backward only.  0: gradient algebra in float, operation by operation as the reference
+                            * writes it (the restatement).  1: the same formulas in double on the same fp32 inputs,
+                            * hits and decisions; the difference between the two shows how much of a float gradient
+                            * value is rounding noise of an ill-conditioned formula (grazing hits, sums that cancel) */
     /* inputs */
     const float *ray_o, *ray_d;   /* (H,W,3) */
     const float *vertices;        /* (4P,3) */
@@ -79,6 +83,11 @@ typedef struct OracleParams {
     float *dL_dshs;                                   /* (P,M,3) */
     float *dL_dcolors, *dL_dothers, *dL_dopacities;   /* (P,3) (P,aux) (P,1) */
     float *dL_dscales, *dL_drotations;                /* (P,2) (P,4) */
+    /* optional, backward with grad_f64 only (all six or none): per element, the summed first-order change of the
+     * geometric gradients when the rounded intermediates of the plane-hit chain (v1 - o, n.(v1-o), n.d) move by one
+     * unit of fp32 rounding of their operands; how far two correct fp32 evaluations of the reference's formula can
+     * be apart on that element.  Shapes as the gradients they belong to. */
+    float *noise_ray_o, *noise_ray_d, *noise_means3D, *noise_grads3D, *noise_scales, *noise_rotations;
 } OracleParams;
 
 /* Both return 0 on success, nonzero on a malformed request. */
@@ -92,6 +101,9 @@ void oracle_quat_to_rows(const float *rot, float *R /* 9, row-major rows u,v,n *
 /* Ray/quad test.  Returns 1 and fills t, tri (0/1) on a hit. */
 int oracle_ray_quad(const float *o, const float *d, const float *A, const float *B, const float *C,
                     const float *Dv, float *t, int *tri);
+/* The three helpers of the reflection chain rule (auxiliary.h:111-121,234-252): which = 0 dnormvdv(v=a, dv=g),
+ * 1 ddotndndn(n=a, d=b, g), 2 ddotndndd(n=a, d=b, g). */
+void oracle_reflection_vjp(int which, const float *a, const float *b, const float *g, float *out);
 /* k nearest hits of one ray: fills up to 16 (t, idx) pairs, returns the admission count. */
 int oracle_k_nearest(const OracleParams *p, const float *o, const float *d, float *t16, uint32_t *idx16);
 int oracle_num_threads(void);

@@ -24,7 +24,7 @@ class OracleParams(C.Structure):
         [(n, C.c_int32) for n in ("P", "H", "W", "D", "M", "aux", "mtd_alloc", "training", "start_from_first",
                                   "max_trace_depth")]
         + [("specular_threshold", C.c_float)]
-        + [(n, C.c_int32) for n in ("hit_mode", "literal_stale", "n_threads")]
+        + [(n, C.c_int32) for n in ("hit_mode", "literal_stale", "n_threads", "grad_f64")]
         + [("ray_o", _FP), ("ray_d", _FP), ("vertices", _FP), ("faces", _IP)]
         + [(n, _FP) for n in ("background", "means3D", "shs", "colors_precomp", "others_precomp", "opacities",
                               "scales", "rotations")]
@@ -34,6 +34,8 @@ class OracleParams(C.Structure):
         + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
         + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
                               "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
+        + [(n, _FP) for n in ("noise_ray_o", "noise_ray_d", "noise_means3D", "noise_grads3D", "noise_scales",
+                              "noise_rotations")]
     )
 
 
@@ -63,6 +65,8 @@ def lib():
         L.oracle_quat_to_rows.argtypes = [_FP, _FP]
         L.oracle_quat_to_rows.restype = None
         L.oracle_ray_quad.argtypes = [_FP] * 6 + [_FP, _IP]
+        L.oracle_reflection_vjp.argtypes = [C.c_int, _FP, _FP, _FP, _FP]
+        L.oracle_reflection_vjp.restype = None
         L.oracle_k_nearest.argtypes = [C.POINTER(OracleParams), _FP, _FP, _FP, C.POINTER(C.c_uint32)]
         _lib = L
     return _lib
@@ -146,9 +150,12 @@ def forward(sc, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0, coun
     return out
 
 
-def backward(sc, fwd, grads, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0):
+def backward(sc, fwd, grads, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0, grad_f64=False, noise=False):
     """Run the oracle backward.  `fwd` is forward()'s dict; `grads` maps rgb/dpt/acc/norm/aux (dist optional)
-    to upstream gradients.  Returns the gradient dict."""
+    to upstream gradients.  Returns the gradient dict.  `grad_f64`: evaluate the gradient algebra in double on
+    the same fp32 inputs and decisions; `noise` (implies grad_f64): also return, under "noise", a dict with the
+    rounding sensitivity of ray_o, ray_d, means3D, grads3D, scales, rotations (see surfel_oracle.h)."""
+    grad_f64 = grad_f64 or noise
     H, W, P = sc.H, sc.W, sc.P
     g = {k: _f32(v) for k, v in grads.items()}
     for k, ch in (("rgb", 3), ("dpt", 1), ("acc", 1), ("norm", 3), ("dist", 1), ("aux", sc.aux)):
@@ -162,6 +169,7 @@ def backward(sc, fwd, grads, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_th
         "scales": np.zeros((P, 2), np.float32), "rotations": np.zeros((P, 4), np.float32),
     }
     p = sc.params(hit_mode, literal_stale, n_threads)
+    p.grad_f64 = int(bool(grad_f64))
     keep = [_f32(fwd[k]) for k in ("rgb", "dpt", "acc", "norm", "dist", "aux", "mid")]
     p.out_rgb, p.out_dpt, p.out_acc, p.out_norm, p.out_dist, p.out_aux, p.mid_val = [_fp(a) for a in keep]
     p.dL_drgb, p.dL_ddpt, p.dL_dacc = _fp(g["rgb"]), _fp(g["dpt"]), _fp(g["acc"])
@@ -170,6 +178,12 @@ def backward(sc, fwd, grads, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_th
     p.dL_dmeans3D, p.dL_dgrads3D, p.dL_dshs = _fp(out["means3D"]), _fp(out["grads3D"]), _fp(out["shs"])
     p.dL_dcolors, p.dL_dothers = _fp(out["colors_precomp"]), _fp(out["others_precomp"])
     p.dL_dopacities, p.dL_dscales, p.dL_drotations = _fp(out["opacities"]), _fp(out["scales"]), _fp(out["rotations"])
+    if noise:
+        nz = {k: np.zeros_like(out[k]) for k in ("ray_o", "ray_d", "means3D", "grads3D", "scales", "rotations")}
+        p.noise_ray_o, p.noise_ray_d = _fp(nz["ray_o"]), _fp(nz["ray_d"])
+        p.noise_means3D, p.noise_grads3D = _fp(nz["means3D"]), _fp(nz["grads3D"])
+        p.noise_scales, p.noise_rotations = _fp(nz["scales"]), _fp(nz["rotations"])
+        out["noise"] = nz
     secs = C.c_double(0.0)
     p.trace_seconds = C.pointer(secs)
     rc = lib().oracle_trace_backward(C.byref(p))
@@ -214,6 +228,14 @@ def ray_quad(o, d, A, B, Cv, Dv):
     tri = C.c_int32(0)
     hit = lib().oracle_ray_quad(*[_fp(a) for a in arrs], C.byref(t), C.byref(tri))
     return bool(hit), t.value, tri.value
+
+
+def reflection_vjp(which, a, b, g):
+    """which: 'dnormvdv' (a = v), 'ddotndndn' (a = n, b = d), 'ddotndndd' (a = n, b = d); g = incoming gradient."""
+    a, b, g = _f32(a), _f32(b), _f32(g)
+    out = np.zeros(3, np.float32)
+    lib().oracle_reflection_vjp({"dnormvdv": 0, "ddotndndn": 1, "ddotndndd": 2}[which], _fp(a), _fp(b), _fp(g), _fp(out))
+    return out
 
 
 def num_threads():

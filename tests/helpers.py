@@ -74,12 +74,80 @@ def assert_forward_exact(gpu, ref, skip=("wet",)):
     assert np.array_equal(gpu["dist"], ref["dist"][..., :1])
 
 
-def assert_close_sum(a, b, rel, name):
-    """Atomically accumulated sums: order differs, so compare against the largest magnitude (north star: 1e-3)."""
+NOISE_FACTOR = 4.0
+
+
+def _report(name, a, b, err, tol, bad, noisy):
+    k = np.unravel_index(np.argmax(err / np.maximum(tol, 1e-300)), err.shape)
+    return ("%s: %d of %d elements off (%d of them carry a rounding-noise allowance); worst at %s: got %.9g, "
+            "want %.9g (|diff| %.3g, allowed %.3g)" % (name, bad.sum(), bad.size, (bad & noisy).sum(), k, a[k], b[k],
+                                                       err[k], tol[k]))
+
+
+def assert_close_sum(a, b, rel, name, noise=None, max_noisy=0.02):
+    """Sums accumulated in a different order on the two sides (atomics on the GPU, double accumulators in the
+    oracle): ELEMENT-WISE |a - b| <= rel * |b| + floor + NOISE_FACTOR * noise.
+    floor: rel/20 of the root-mean-square of the channel's nonzero entries (a sum that cancels keeps the rounding
+    of its summands while its value shrinks; the columns of one tensor can differ by orders of magnitude).
+    noise: what fp32 rounding alone does to this element of the reference's formula, from the oracle: |b - b64|
+    (b64 = its gradient algebra evaluated in double on the same fp32 inputs and decisions) plus, for the
+    geometric gradients, its first-order sensitivity to one unit of rounding in the plane-hit chain (a grazing
+    hit at 50 m divides a difference of two 50 m vectors by n.d twice: one ulp in t = n.(v1-o)/n.d moves such an
+    element by tens of per cent).  No fp32 implementation, the reference's included, is closer to another than that.
+    At most `max_noisy` of the elements may owe their pass to the noise term."""
     assert a.shape == b.shape, (name, a.shape, b.shape)
-    scale = max(float(np.abs(b).max()), 1e-30)
-    err = float(np.abs(a - b).max()) / scale
-    assert err <= rel, "%s: max error %.3g of max |ref| %.3g exceeds %.1g" % (name, err, scale, rel)
+    a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    flat_b = b64.reshape(-1, b64.shape[-1]) if b64.ndim > 1 else b64.reshape(-1, 1)
+    flat_a = a64.reshape(flat_b.shape)
+    assert np.isfinite(flat_a).all() == np.isfinite(flat_b).all(), name
+    live = flat_b != 0
+    rms = np.sqrt((flat_b ** 2).sum(0) / np.maximum(live.sum(0), 1))
+    base = rel * np.abs(flat_b) + rel / 20 * rms[None, :]
+    extra = 0.0 if noise is None else NOISE_FACTOR * np.asarray(noise, np.float64).reshape(flat_b.shape)
+    err = np.abs(flat_a - flat_b)
+    tol = base + extra
+    bad = err > tol
+    noisy = (err > base)
+    if bad.any():
+        raise AssertionError(_report(name, flat_a, flat_b, err, tol, bad, noisy))
+    assert noisy.mean() <= max_noisy, "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean())
+
+
+def assert_close_rays(a, b, rel, name, noise=None, max_noisy=0.02):
+    """Per-ray gradients are plain stores (no atomics): element-wise |a - b| <= rel * |b| + rel/10 * (largest
+    component of that ray's gradient) + NOISE_FACTOR * noise (see assert_close_sum)."""
+    assert a.shape == b.shape, (name, a.shape, b.shape)
+    a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    row = np.abs(b64).max(-1, keepdims=True)
+    base = rel * np.abs(b64) + rel / 10 * row + 1e-30
+    extra = 0.0 if noise is None else NOISE_FACTOR * np.asarray(noise, np.float64)
+    err, tol = np.abs(a64 - b64), base + extra
+    bad = err > tol
+    noisy = err > base
+    if bad.any():
+        raise AssertionError(_report(name, a64, b64, err, tol, bad, noisy))
+    assert noisy.mean() <= max_noisy, "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean())
+
+
+def assert_gradients(got, ref32, ref64, rel, tag=""):
+    """Every gradient tensor of `got` (GPU) against the oracle's (`ref32`).  `ref64` = oracle.backward(...,
+    noise=True): its double-precision values and its sensitivity estimate together give the rounding-noise allowance."""
+    est = {} if ref64 is None else ref64.get("noise", {})
+    for k, want in ref32.items():
+        if k == "noise":
+            continue
+        if got.get(k) is None:
+            assert k in ("shs", "colors_precomp", "others_precomp"), k
+            continue
+        if np.abs(want).max() == 0 and k not in est:
+            assert np.abs(got[k]).max() == 0, k
+            continue
+        noise = None
+        if ref64 is not None:
+            noise = np.abs(want.astype(np.float64) - ref64[k].astype(np.float64))
+            if k in est:
+                noise = noise + est[k].astype(np.float64)
+        (assert_close_rays if k in ("ray_o", "ray_d") else assert_close_sum)(got[k], want, rel, tag + k, noise=noise)
 
 
 GRAD_REL = 1e-3   # north star: gradients within 1e-3 relative

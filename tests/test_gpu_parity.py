@@ -1,19 +1,21 @@
 """Parity of the HIP path (through the public API and the C ABI underneath) with the CPU oracle on the
 same seeded inputs.  Bar: per-ray forward outputs bit-identical (both sides run the same sequence of
-unfused fp32 operations; the north star asks for 1e-4 absolute), atomically accumulated sums and all
-gradients within 1e-3 of the largest reference magnitude (north star: 1e-3 relative)."""
+unfused fp32 operations; the north star asks for 1e-4 absolute); atomically accumulated sums and all
+gradients element-wise within 1e-3 relative (north star: 1e-3 relative) plus a floor for sums that cancel
+(helpers.assert_close_sum / assert_close_rays)."""
 import numpy as np
 import pytest
 import torch
 
 import dst_scenes as S
-from helpers import (GRAD_REL, assert_close_sum, assert_forward_exact, gpu_trace, oracle_scene, to_numpy, upstream)
+from helpers import (GRAD_REL, assert_close_sum, assert_forward_exact, assert_gradients, gpu_trace, oracle_scene,
+                     to_numpy, upstream)
 
 pytestmark = pytest.mark.gpu
 
 
-def check_case(oracle, tracer, scene, ray_o, ray_d, acc_grad=True, grads=True, **kw):
-    """Forward + backward on both sides and compare everything."""
+def check_case(oracle, tracer, scene, ray_o, ray_d, acc_grad=True, grads=True, skip=(), **kw):
+    """Forward + backward on both sides and compare everything (but the gradient tensors named in `skip`)."""
     H, W = ray_o.shape[:2]
     s = oracle_scene(oracle, scene, ray_o, ray_d, **kw)
     ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
@@ -22,15 +24,11 @@ def check_case(oracle, tracer, scene, ray_o, ray_d, acc_grad=True, grads=True, *
     assert_forward_exact(out, ref)
     assert_close_sum(out["wet"], ref["wet"], 1e-5, "wet")
     if grads:
-        refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
-        for k, want in refg.items():
-            if g.get(k) is None:
-                assert k in ("shs", "colors_precomp", "others_precomp"), k
-                continue
-            if np.abs(want).max() == 0:
-                assert np.abs(g[k]).max() == 0, k
-                continue
-            assert_close_sum(g[k], want, GRAD_REL, k)
+        ugn = {k: v.numpy() for k, v in ug.items()}
+        refg = oracle.backward(s, ref, ugn, oracle.HITS_BVH_LEXI)
+        refg64 = oracle.backward(s, ref, ugn, oracle.HITS_BVH_LEXI, noise=True)
+        assert_gradients(g, {k: v for k, v in refg.items() if k not in skip}, refg64, GRAD_REL)
+        ref["grads_gpu"], ref["grads_ref"] = g, refg
     return ref, out
 
 
@@ -135,8 +133,14 @@ def test_coplanar_ties_and_dense_stacks(oracle, tracer):
     o = torch.stack(torch.meshgrid(torch.linspace(-0.4, 0.4, 24), torch.linspace(-0.4, 0.4, 24), indexing="ij"), -1)
     o = torch.cat([o, torch.full((24, 24, 1), 3.0)], -1).contiguous()
     d = torch.tensor([0.0, 0.0, -1.0]).expand(24, 24, 3).contiguous()
-    ref, _ = check_case(oracle, tracer, sc, o, d)
+    # The quads are axis-aligned (identity quaternions) and the rays run along -z: the rotation gradient is zero by
+    # symmetry, what either side returns for it is the rounding left over from terms of the size of the scale
+    # gradient that cancel, so it is compared against that size instead of element by element.
+    ref, _ = check_case(oracle, tracer, sc, o, d, skip=("rotations",))
     assert ref["n_proc"].max() >= 16
+    big = np.abs(ref["grads_ref"]["scales"]).max()
+    assert np.abs(ref["grads_ref"]["rotations"]).max() <= 1e-6 * big
+    assert np.abs(ref["grads_gpu"]["rotations"]).max() <= 1e-6 * big
 
 
 def test_refit_equals_rebuild(oracle, tracer):
@@ -206,6 +210,7 @@ def test_backward_replays_the_forward_hit_record_or_retraces(oracle, tracer):
     ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
     ug = upstream(64, 64, 2)
     refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
+    refg64 = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI, noise=True)
     ctx = tracer.optix_context
     saved = ctx.record_blocks_per_wave
     try:
@@ -213,8 +218,7 @@ def test_backward_replays_the_forward_hit_record_or_retraces(oracle, tracer):
             ctx.record_blocks_per_wave = estimate
             out, g = gpu_trace(tracer, sc, o, d, upstream=ug)
             assert_forward_exact(out, ref)
-            for k in ("ray_o", "ray_d", "means3D", "grads3D", "shs", "opacities", "scales", "rotations"):
-                assert_close_sum(g[k], refg[k], GRAD_REL, k)
+            assert_gradients(g, refg, refg64, GRAD_REL)
         torch.cuda.synchronize()
         ctx.update_record_estimate()
         assert ctx.record_blocks_per_wave > 1.0   # learnt from the overflow, without the backward call waiting for it
@@ -243,6 +247,7 @@ def test_raw_launcher_calls_without_a_record(oracle, tracer):
     s = oracle_scene(oracle, sc, o, d)
     ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
     refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
+    refg64 = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI, noise=True)
     np.testing.assert_array_equal(fwd[0].cpu().numpy(), ref["rgb"])
     # hit counts: entries evaluated and hits composited, summed over the rays, are the oracle's exactly
     counters = torch.zeros(2, dtype=torch.int64, device=dev)
@@ -250,7 +255,6 @@ def test_raw_launcher_calls_without_a_record(oracle, tracer):
     assert counters.tolist() == [int(ref["n_proc"].sum()), int(ref["n_con"].sum())]
     names = ("ray_o", "ray_d", "means3D", "grads3D", None, "shs", "colors_precomp", None, "opacities", "scales",
              "rotations", None)
-    for t, k in zip(bwd, names):
-        if k is not None:
-            assert_close_sum(t.cpu().numpy(), refg[k], GRAD_REL, k)
+    got = {k: t.cpu().numpy() for t, k in zip(bwd, names) if k is not None}
+    assert_gradients(got, {k: refg[k] for k in got}, refg64, GRAD_REL)
     assert bwd[4].abs().max() == 0 and bwd[11].shape == (3000, 9) and bwd[11].abs().max() == 0

@@ -5,12 +5,19 @@ The reference's backward deviates from the true gradient in documented ways; the
 the subset where it does not, or against a forward adjusted to express the deviation:
   - background: mid_val's colour already contains T*bg and backward adds the background term again
     (backward.cu:545-548), which is the exact gradient of a forward whose background weight is doubled;
-  - accumulated weight: W is never accumulated (backward.cu:568), so dL/dacc flows wrongly -> not fed here;
+  - accumulated weight: W is never accumulated (backward.cu:568), so the gradient of acc w.r.t. a hit's alpha is
+    T_i - acc/(1-alpha_i) instead of T_i - (acc - W_i)/(1-alpha_i); that is the exact gradient of the surrogate
+    acc - sum_i stopgrad(W_i/(1-alpha_i)) * alpha_i, which is what the dL/dacc test differentiates;
+  - reflection origin: forward offsets the next origin by START_OFFSET (0.06) along the reflected direction, backward
+    chains STEP_EPSILON (1e-5) instead (backward.cu:782 vs forward.cu:422): the exact gradient of a forward whose
+    next origin is E + 1e-5 d' + stopgrad((0.06 - 1e-5) d');
   - SH mode overwrites the ray-direction gradient per hit (backward.cu:165,631) -> ray_d is compared in
     colour mode only;
   - quaternion gradients omit the normalisation Jacobian (auxiliary.h:433-477) -> compared after
     projecting the oracle's gradient with (I - q q^T) for unit q.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -100,7 +107,7 @@ def forward64(ro, rd, means, scales, quats, opac, bg, colors=None, shs=None, oth
         oth = others[None].expand(ro.shape[0], -1, -1)
         aux = (w[..., None] * torch.gather(oth, 1, order[..., None].expand(-1, -1, others.shape[1]))).sum(1)
     edge = torch.where(in0 | in1, torch.where(in0, m0, m1), torch.minimum(m0, m1))
-    info = {"n_con": (w > 0).sum(1), "edge_margin": torch.where(t > 0, edge, torch.ones_like(edge)).min(),
+    info = {"n_con": (w > 0).sum(1), "w": w, "alpha": a_s, "acc": w.sum(1), "edge_margin": torch.where(t > 0, edge, torch.ones_like(edge)).min(),
             "thresh_margin": torch.where(hit, (alpha - 1 / 255).abs(), torch.ones_like(alpha)).min()}
     return rgb, dpt, nrm, aux, info
 
@@ -306,3 +313,280 @@ def test_second_bounce_gradients_match_autograd_with_the_reflected_rays_held_fix
     check("colours of all", got["colors_precomp"], leaf["colors_precomp"].grad, slice(0, PA + PB))
     # the specular channel of the mirror weighs the two bounces against each other: d out / d O0 = C1 - C0
     check("aux channels of all", got["others_precomp"], leaf["others_precomp"].grad, slice(0, PA + PB))
+
+
+def acc_surrogate(info):
+    """acc as the reference's backward differentiates it (W never accumulated, backward.cu:568)."""
+    w, a = info["w"], info["alpha"]
+    W = torch.cumsum(w, dim=1)
+    return info["acc"] - ((W / (1 - a)).detach() * a).sum(1)
+
+
+def reference_like_loss(ro64, rd64, leaf, bg64, up, args, bg_weight=2.0, with_acc=True):
+    rgb, dpt, nrm, aux, info = forward64(ro64, rd64, leaf["means3D"], leaf["scales"], leaf["rotations"],
+                                         leaf["opacities"], bg64, bg_weight=bg_weight, **args)
+    loss = (rgb * up["rgb"].double()).sum() + (dpt * up["dpt"].double()[:, 0]).sum() + \
+        (nrm * up["norm"].double()).sum() + (aux * up["aux"].double()).sum()
+    if with_acc:
+        loss = loss + (acc_surrogate(info) * up["acc"].double()[:, 0]).sum()
+    return loss
+
+
+def relcheck(name, mine, want, rel=3e-4, rows=slice(None)):
+    want = want.numpy()[rows] if hasattr(want, "numpy") else np.asarray(want)[rows]
+    mine = np.asarray(mine, np.float64).reshape(-1, *want.shape[1:])[rows] if want.ndim > 1 else np.asarray(mine, np.float64).reshape(-1)[rows]
+    scale = np.abs(want).max()
+    assert scale > 0, name
+    err = np.abs(mine.reshape(want.shape) - want).max() / scale
+    if os.environ.get("DST_SHOW_ERR"):
+        print("%-14s relative error %.3g" % (name, err))
+    assert err < rel, "%s: relative error %.3g" % (name, err)
+
+
+@pytest.mark.parametrize("seed,only_acc", [(21, True), (22, False)])
+def test_dL_dacc_flow_matches_autograd_of_the_surrogate(oracle, seed, only_acc):
+    """Pins the dL/dacc path of bounce_backward: upstream gradient on acc alone, then mixed with the others."""
+    sc, ro, rd, up = make_case(seed, sh=False)
+    R = ro.shape[0]
+    gen = torch.Generator().manual_seed(seed + 100)
+    up["acc"] = torch.randn(R, 1, generator=gen)
+    if only_acc:
+        up = {k: (v if k == "acc" else torch.zeros_like(v)) for k, v in up.items()}
+    s = oracle_scene(oracle, sc, ro.reshape(1, R, 3), rd.reshape(1, R, 3))
+    fwd = oracle.forward(s, oracle.HITS_BRUTE_LEXI)
+    got = oracle.backward(s, fwd, {k: v.reshape(1, R, -1).numpy() for k, v in up.items()}, oracle.HITS_BRUTE_LEXI)
+    leaf = {k: sc[k].double().requires_grad_(True) for k in sc if k not in ("vertices", "faces")}
+    ro64, rd64 = ro.double().requires_grad_(True), rd.double().requires_grad_(True)
+    args = dict(colors=leaf.get("colors_precomp"), others=leaf.get("others_precomp"))
+    bg64 = torch.zeros(3, dtype=torch.float64)
+    _, _, _, _, info = forward64(ro64, rd64, leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["opacities"],
+                                 bg64, **args)
+    np.testing.assert_allclose(fwd["acc"].reshape(R), info["acc"].detach().numpy(), atol=2e-5)
+    np.testing.assert_array_equal(fwd["n_con"].reshape(R), info["n_con"].numpy())
+    assert (info["n_con"] >= 2).sum() > R // 2      # W_i differs from 0 and from acc on most rays
+    reference_like_loss(ro64, rd64, leaf, bg64, up, args).backward()
+    relcheck("means3D", got["means3D"], leaf["means3D"].grad)
+    relcheck("scales", got["scales"], leaf["scales"].grad)
+    relcheck("opacities", got["opacities"], leaf["opacities"].grad)
+    relcheck("ray_o", got["ray_o"], ro64.grad)
+    relcheck("ray_d", got["ray_d"], rd64.grad)
+    q = sc["rotations"].double().numpy()
+    proj = got["rotations"].astype(np.float64) - q * (q * got["rotations"]).sum(-1, keepdims=True)
+    relcheck("rotations", proj, leaf["rotations"].grad)
+    # the true gradient of acc is a different vector: the surrogate is not a no-op
+    leaf2 = {k: sc[k].double().requires_grad_(True) for k in sc if k not in ("vertices", "faces")}
+    _, _, _, _, info2 = forward64(ro.double(), rd.double(), leaf2["means3D"], leaf2["scales"], leaf2["rotations"],
+                                  leaf2["opacities"], bg64, colors=leaf2["colors_precomp"], others=leaf2["others_precomp"])
+    (info2["acc"] * up["acc"].double()[:, 0]).sum().backward()
+    if only_acc:
+        true_g = leaf2["opacities"].grad.numpy()
+        assert np.abs(true_g - got["opacities"]).max() > 0.05 * np.abs(true_g).max()
+
+
+def test_reflection_helpers_are_the_jacobians_they_claim(oracle):
+    """dnormvdv = J_normalize(v)^T g;  ddotndndn / ddotndndd = vjp of f(n, d) = (n.d) n w.r.t. n / d
+    (auxiliary.h:111-121, 234-252)."""
+    gen = torch.Generator().manual_seed(31)
+    for _ in range(20):
+        v = torch.randn(3, generator=gen, dtype=torch.float64) * 3
+        d = torch.randn(3, generator=gen, dtype=torch.float64)
+        g = torch.randn(3, generator=gen, dtype=torch.float64)
+        v1 = v.clone().requires_grad_(True)
+        ((v1 / v1.norm()) * g).sum().backward()
+        np.testing.assert_allclose(oracle.reflection_vjp("dnormvdv", v.numpy(), d.numpy(), g.numpy()), v1.grad.numpy(),
+                                   rtol=2e-5, atol=1e-6)
+        n = (v / v.norm()).clone().requires_grad_(True)
+        d1 = d.clone().requires_grad_(True)
+        (((n * d1).sum() * n) * g).sum().backward()
+        np.testing.assert_allclose(oracle.reflection_vjp("ddotndndn", n.detach().numpy(), d.numpy(), g.numpy()),
+                                   n.grad.numpy(), rtol=2e-5, atol=1e-6)
+        np.testing.assert_allclose(oracle.reflection_vjp("ddotndndd", n.detach().numpy(), d.numpy(), g.numpy()),
+                                   d1.grad.numpy(), rtol=2e-5, atol=1e-6)
+
+
+def mirror_scene(seed, PA=40, PB=60, R=48):
+    """A "mirror" cluster A around z = 0 facing a camera at z = 2 and a cluster B above the camera that only the
+    reflected rays can reach."""
+    gen = torch.Generator().manual_seed(seed)
+    meansA = torch.cat([(torch.rand(PA, 2, generator=gen) * 2 - 1) * 0.45, 0.02 * torch.randn(PA, 1, generator=gen)], -1)
+    qA = torch.tensor([1.0, 0.0, 0.0, 0.0]) + 0.08 * torch.randn(PA, 4, generator=gen)
+    meansB = torch.cat([(torch.rand(PB, 2, generator=gen) * 2 - 1) * 0.9, 3.2 + 0.3 * torch.rand(PB, 1, generator=gen)], -1)
+    qB = torch.randn(PB, 4, generator=gen)
+    q = torch.cat([qA, qB])
+    q = q / q.norm(dim=-1, keepdim=True)
+    scales = torch.cat([torch.exp(-1.6 + 0.2 * torch.randn(PA, 2, generator=gen)),
+                        torch.exp(-1.3 + 0.3 * torch.randn(PB, 2, generator=gen))])
+    others = torch.rand(PA + PB, 2, generator=gen)
+    others[:PA, 0] = 0.5 + 0.4 * others[:PA, 0]
+    sc = {"means3D": torch.cat([meansA, meansB]), "scales": scales, "rotations": q,
+          "opacities": torch.sigmoid(1.0 + torch.randn(PA + PB, 1, generator=gen)),
+          "colors_precomp": torch.rand(PA + PB, 3, generator=gen), "others_precomp": others}
+    sc = {k: v.float().contiguous() for k, v in sc.items()}
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    ro = torch.tensor([0.0, 0.0, 2.0]) + 0.03 * torch.randn(R, 3, generator=gen)
+    target = torch.cat([(torch.rand(R, 2, generator=gen) * 2 - 1) * 0.3, torch.zeros(R, 1)], -1)
+    rd = target - ro
+    rd = (rd / rd.norm(dim=-1, keepdim=True)).float().contiguous()
+    up = {"rgb": torch.randn(R, 3, generator=gen), "dpt": torch.randn(R, 1, generator=gen),
+          "norm": torch.randn(R, 3, generator=gen), "aux": torch.randn(R, 2, generator=gen),
+          "acc": torch.randn(R, 1, generator=gen)}
+    return sc, ro.float().contiguous(), rd, up
+
+
+@pytest.mark.parametrize("seed", [42, 43, 44, 45])
+def test_full_two_bounce_chain_matches_autograd_with_the_reflected_rays_free(oracle, seed):
+    """Pins the reflection-geometry chain of path_backward (backward.cu:700-790): the reflected ray of bounce 1 is a
+    differentiable function of bounce 0's depth, normal, origin and direction,
+        E = o + D d,  n = N/|N|,  d' = d - 2 (n.d) n,  o' = E + 1e-5 d' + stopgrad((0.06 - 1e-5) d'),
+    and the float64 model renders bounce 1 from (o', d').  Every gradient the oracle returns, for every surfel and
+    every ray, is compared with autograd of that model (the acc output through its surrogate)."""
+    sc, ro, rd, up = mirror_scene(seed)
+    R, PA = ro.shape[0], 40
+    s = oracle_scene(oracle, sc, ro.reshape(1, R, 3), rd.reshape(1, R, 3), max_trace_depth=1, specular_threshold=0.0)
+    fwd = oracle.forward(s, oracle.HITS_BRUTE_LEXI)
+    got = oracle.backward(s, fwd, {k: v.reshape(1, R, -1).numpy() for k, v in up.items()}, oracle.HITS_BRUTE_LEXI)
+    mid = torch.from_numpy(fwd["mid"].reshape(R, 2, 16)).double()
+    bounced = mid[:, 1, 3:6].norm(dim=-1) > 0
+
+    leaf = {k: sc[k].double().requires_grad_(True) for k in sc if k not in ("vertices", "faces")}
+    ro64, rd64 = ro.double().requires_grad_(True), rd.double().requires_grad_(True)
+    zero_bg = torch.zeros(3, dtype=torch.float64)
+    args = dict(colors=leaf["colors_precomp"], others=leaf["others_precomp"])
+    geo = (leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["opacities"], zero_bg)
+    C0, D0, N0, O0, info0 = forward64(ro64, rd64, *geo, **args)
+    hit0 = info0["n_con"] > 0
+    np.testing.assert_array_equal(bounced.numpy(), hit0.numpy())     # threshold 0: every ray that hits bounces
+    assert hit0.sum() > R // 2
+    Nsafe = torch.where(hit0[:, None], N0, torch.tensor([0.0, 0.0, 1.0], dtype=torch.float64).expand(R, 3))
+    n = Nsafe / Nsafe.norm(dim=-1, keepdim=True)
+    d1 = rd64 - 2 * (n * rd64).sum(-1, keepdim=True) * n
+    E = ro64 + D0[:, None] * rd64
+    o1 = E + 1e-5 * d1 + ((0.06 - 1e-5) * d1).detach()
+    np.testing.assert_allclose(mid[bounced][:, 1, 0:3].numpy(), o1[bounced].detach().numpy(), atol=2e-5)
+    np.testing.assert_allclose(mid[bounced][:, 1, 3:6].numpy(), d1[bounced].detach().numpy(), atol=2e-5)
+    C1, _, _, _, info1 = forward64(o1, d1, *geo, near=0.06, **args)
+    C1 = torch.where(hit0[:, None], C1, torch.zeros_like(C1))
+    s0 = O0[:, :1]
+    out = C0 * (1 - s0) + C1 * s0
+    np.testing.assert_allclose(fwd["rgb"].reshape(R, 3), out.detach().numpy(), atol=3e-5)
+    n1 = torch.where(hit0, info1["n_con"], torch.zeros_like(info1["n_con"]))
+    np.testing.assert_array_equal(fwd["n_con"].reshape(R), (info0["n_con"] + n1).numpy())
+    assert n1.sum() > R
+
+    loss = (out * up["rgb"].double()).sum() + (D0 * up["dpt"].double()[:, 0]).sum() + \
+        (N0 * up["norm"].double()).sum() + (O0 * up["aux"].double()).sum() + \
+        (acc_surrogate(info0) * up["acc"].double()[:, 0]).sum()
+    loss.backward()
+    # the chain really carries weight: with the reflected rays held fixed the mirror's gradients are different
+    relcheck("means3D", got["means3D"], leaf["means3D"].grad)
+    relcheck("scales", got["scales"], leaf["scales"].grad)
+    relcheck("opacities", got["opacities"], leaf["opacities"].grad)
+    relcheck("colours", got["colors_precomp"], leaf["colors_precomp"].grad)
+    relcheck("aux channels", got["others_precomp"], leaf["others_precomp"].grad)
+    qn = sc["rotations"].double().numpy()
+    proj = got["rotations"].astype(np.float64) - qn * (qn * got["rotations"]).sum(-1, keepdims=True)
+    relcheck("rotations", proj, leaf["rotations"].grad)
+    relcheck("ray_o", got["ray_o"], ro64.grad)
+    relcheck("ray_d", got["ray_d"], rd64.grad)
+
+
+def test_three_bounce_weights_and_chained_reflections(oracle):
+    """Depth 2 (beyond the reference's shipped MAX_TRACE_DEPTH = 1; the oracle follows the reference's loop as if
+    compiled for it).  Two facing mirrors: camera -> A -> B -> A.  On rays that are traced through all three
+    bounces the reference's weights are the true ones (g C_i: f_i prod s_j; d out/d s_1) except for d out/d s_0,
+    where its running colour is updated with a specular product that was already divided (backward.cu:762-774):
+    it yields s_1 (C_2 - C_1) + (C_1 - C_0)/s_0 instead of s_1 (C_2 - C_1) + (C_1 - C_0).  That difference is added
+    to the model as a stop-gradient coefficient on s_0; everything else (per-bounce colour weights, the gradient
+    w.r.t. s_1, two chained reflections) is autograd of the float64 forward.  Rays that end early get no upstream
+    gradient here (the reference scales them by a skipped specular, backward.cu:724-725)."""
+    gen = torch.Generator().manual_seed(51)
+    PA, PB, R = 50, 70, 40
+    meansA = torch.cat([(torch.rand(PA, 2, generator=gen) * 2 - 1) * 0.5, 0.02 * torch.randn(PA, 1, generator=gen)], -1)
+    meansB = torch.cat([(torch.rand(PB, 2, generator=gen) * 2 - 1) * 0.9, 3.4 + 0.02 * torch.randn(PB, 1, generator=gen)], -1)
+    q = torch.tensor([1.0, 0.0, 0.0, 0.0]) + 0.05 * torch.randn(PA + PB, 4, generator=gen)
+    q = q / q.norm(dim=-1, keepdim=True)
+    scales = torch.cat([torch.exp(-1.5 + 0.2 * torch.randn(PA, 2, generator=gen)),
+                        torch.exp(-1.2 + 0.2 * torch.randn(PB, 2, generator=gen))])
+    others = torch.rand(PA + PB, 2, generator=gen)
+    others[:, 0] = 0.5 + 0.4 * others[:, 0]
+    sc = {"means3D": torch.cat([meansA, meansB]), "scales": scales, "rotations": q,
+          "opacities": torch.sigmoid(0.5 + torch.randn(PA + PB, 1, generator=gen)),
+          "colors_precomp": torch.rand(PA + PB, 3, generator=gen), "others_precomp": others}
+    sc = {k: v.float().contiguous() for k, v in sc.items()}
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    ro = (torch.tensor([0.0, 0.0, 2.0]) + 0.03 * torch.randn(R, 3, generator=gen)).float().contiguous()
+    target = torch.cat([(torch.rand(R, 2, generator=gen) * 2 - 1) * 0.25, torch.zeros(R, 1)], -1)
+    rd = target - ro
+    rd = (rd / rd.norm(dim=-1, keepdim=True)).float().contiguous()
+
+    s = oracle_scene(oracle, sc, ro.reshape(1, R, 3), rd.reshape(1, R, 3), max_trace_depth=2, specular_threshold=0.0)
+    fwd = oracle.forward(s, oracle.HITS_BRUTE_LEXI)
+    mid = torch.from_numpy(fwd["mid"].reshape(R, 3, 16)).double()
+    full = mid[:, 2, 3:6].norm(dim=-1) > 0                      # traced through all three bounces
+    assert full.sum() > R // 2
+    up = {"rgb": torch.randn(R, 3, generator=gen) * full[:, None], "dpt": torch.randn(R, 1, generator=gen) * full[:, None],
+          "norm": torch.randn(R, 3, generator=gen) * full[:, None], "aux": torch.randn(R, 2, generator=gen) * full[:, None]}
+    got = oracle.backward(s, fwd, {k: v.reshape(1, R, -1).numpy() for k, v in up.items()}, oracle.HITS_BRUTE_LEXI)
+
+    leaf = {k: sc[k].double().requires_grad_(True) for k in sc if k not in ("vertices", "faces")}
+    ro64, rd64 = ro.double().requires_grad_(True), rd.double().requires_grad_(True)
+    geo = (leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["opacities"], torch.zeros(3, dtype=torch.float64))
+    args = dict(colors=leaf["colors_precomp"], others=leaf["others_precomp"])
+    o, d, near = ro64, rd64, 0.2
+    Cs, Ss, first, n_total = [], [], None, 0
+    for i in range(3):
+        C, D, N, O, info = forward64(o, d, *geo, near=near, **args)
+        if i == 0:
+            first = (D, N, O)
+        np.testing.assert_allclose(mid[full][:, i, 13:16].numpy(), C[full].detach().numpy(), atol=5e-5)
+        n_total = n_total + info["n_con"]
+        Cs.append(C)
+        Ss.append(O[:, :1])
+        if i < 2:
+            Nsafe = torch.where(full[:, None], N, torch.tensor([0.0, 0.0, 1.0], dtype=torch.float64).expand(R, 3))
+            n = Nsafe / Nsafe.norm(dim=-1, keepdim=True)
+            d_next = d - 2 * (n * d).sum(-1, keepdim=True) * n
+            o = o + D[:, None] * d + 1e-5 * d_next + ((0.06 - 1e-5) * d_next).detach()
+            d, near = d_next, 0.06
+    np.testing.assert_array_equal(fwd["n_con"].reshape(R)[full.numpy()], n_total[full].numpy())
+    s0, s1 = Ss[0], Ss[1]
+    out = Cs[0] * (1 - s0) + s0 * Cs[1] * (1 - s1) + s0 * s1 * Cs[2]
+    np.testing.assert_allclose(fwd["rgb"].reshape(R, 3)[full.numpy()], out[full].detach().numpy(), atol=5e-5)
+    g = up["rgb"].double()
+    quirk = (((Cs[1] - Cs[0]) * (1 / s0 - 1)).detach() * g).sum(-1, keepdim=True) * s0      # see the docstring
+    loss = (out * g).sum() + quirk.sum() + (first[0] * up["dpt"].double()[:, 0]).sum() + \
+        (first[1] * up["norm"].double()).sum() + (first[2] * up["aux"].double()).sum()
+    loss.backward()
+    relcheck("means3D", got["means3D"], leaf["means3D"].grad)
+    relcheck("scales", got["scales"], leaf["scales"].grad)
+    relcheck("opacities", got["opacities"], leaf["opacities"].grad)
+    relcheck("colours", got["colors_precomp"], leaf["colors_precomp"].grad)
+    relcheck("aux channels", got["others_precomp"], leaf["others_precomp"].grad)
+    qn = sc["rotations"].double().numpy()
+    proj = got["rotations"].astype(np.float64) - qn * (qn * got["rotations"]).sum(-1, keepdims=True)
+    relcheck("rotations", proj, leaf["rotations"].grad)
+    relcheck("ray_o", got["ray_o"], ro64.grad)
+    relcheck("ray_d", got["ray_d"], rd64.grad)
+
+
+def test_rounding_sensitivity_estimate_covers_the_float_evaluation_and_stays_small(oracle):
+    """The comparison of the HIP path with the oracle allows each geometric gradient element a multiple of the
+    oracle's sensitivity estimate (helpers.assert_gradients).  Here: that estimate covers what fp32 rounding does
+    to the oracle's own float evaluation (float vs double algebra), on a LiDAR scene (hits 50 m away at grazing
+    angles: many noisy elements) and on the unit-cube scene, where it exceeds the plain 1e-3 relative bound on a
+    small share of the elements only, so the comparison keeps its teeth."""
+    from helpers import NOISE_FACTOR
+    lidar = S.perturb_means(S.scene_lidar(P=60000, seed=0, aux=4), 1)
+    cases = ((lidar, S.rays_lidar(beams=32, azimuths=256), 4, 0.2), (S.scene_cube(P=3000, seed=1), S.rays_cube(48, 48), 2, 0.06))
+    for sc, (o, d), aux, share in cases:
+        up = {k: v.numpy() for k, v in S.upstream_grads(o.shape[0], o.shape[1], aux).items()}
+        s = oracle_scene(oracle, sc, o, d)
+        fwd = oracle.forward(s, oracle.HITS_BVH_LEXI)
+        g32 = oracle.backward(s, fwd, up, oracle.HITS_BVH_LEXI)
+        g64 = oracle.backward(s, fwd, up, oracle.HITS_BVH_LEXI, noise=True)
+        assert fwd["n_con"].sum() > 1000
+        for k in ("scales", "rotations", "means3D", "grads3D", "ray_o"):
+            b, est = g32[k].astype(np.float64), g64["noise"][k].astype(np.float64)
+            diff = np.abs(b - g64[k])
+            assert (diff <= 1e-3 * np.abs(b) + NOISE_FACTOR * est + 1e-6 * np.abs(b).max()).all(), k
+            assert (est > 1e-3 * np.abs(b))[b != 0].mean() < share, k
