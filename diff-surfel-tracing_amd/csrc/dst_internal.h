@@ -49,6 +49,20 @@ struct alignas(16) DstLeaf {
 };
 static_assert(sizeof(DstLeaf) == 80, "leaf records are 20 dwords");
 
+// Cheap conservative stand-in for the exact ray/quad test, one per leaf (same order): the quad as a parallelogram
+// on its mean plane.  A ray whose hit point on that plane has |s|, |r| beyond `lim0` (plus a margin for rounding)
+// cannot pass the exact test; the walk fetches the 80-byte record and runs the exact test only if some lane
+// survives.  c = centroid, n = unit normal, fu/fv = dual vectors of the averaged half edges (s = fu.(P-c),
+// r = fv.(P-c): the corners sit at about (+-1, +-1)), mfu = max(|fu|, |fv|), lim0 = largest |s| or |r| of a
+// corner, a little enlarged, tdev = how far the corners leave the mean plane, enlarged (0 for a planar quad).
+// A degenerate quad gets mfu = inf: every ray survives.
+struct alignas(64) DstLeafPre {
+    float c[3], n[3], fu[3], fv[3];
+    float mfu, lim0, tdev;
+    uint32_t pad;
+};
+static_assert(sizeof(DstLeafPre) == 64, "one 16-dword scalar fetch");
+
 struct DstBounds {          // device-resident reduction targets, order-preserving uint encoding
     uint32_t lo[3], hi[3];  // centroid bounds
     uint32_t max_abs;       // raw bits of a non-negative float: largest |coordinate| of any vertex
@@ -59,6 +73,7 @@ struct DstBounds {          // device-resident reduction targets, order-preservi
 struct DstAccelView {
     const DstWideNode *wide;
     const DstLeaf *leaves;
+    const DstLeafPre *pre;
     const DstBounds *bounds;  // max_abs sizes the conservative slab padding; read on the device so that a
                               // refit never needs a host round trip
     uint32_t root;
@@ -77,6 +92,7 @@ struct dst_ctx {
     DstNode *nodes = nullptr;
     DstWideNode *wide = nullptr;
     DstLeaf *leaves = nullptr;
+    DstLeafPre *pre = nullptr;
     uint32_t *node_parent = nullptr, *leaf_parent = nullptr;  // (parent << 1) | which child
     uint32_t *flags = nullptr;                                // arrival counters of the bottom-up fit
     int32_t *quad_ids = nullptr;                              // 4 vertex ids per surfel (int4)

@@ -294,7 +294,8 @@ __global__ void k_karras(const uint32_t *__restrict__ keys, DstNode *__restrict_
 // Leaf records in Morton order (also the whole of a refit's geometry update).  The plane normals use the
 // fused form the hit test is defined with: cross(x,y).x = fma(x.y, y.z, -(x.z*y.y)), and so on.
 __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
-                            const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves, uint32_t n) {
+                            const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
+                            DstLeafPre *__restrict__ pre, uint32_t n) {
     uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     uint32_t g = sorted_ids[i];
@@ -337,6 +338,59 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
     float4 *dst = reinterpret_cast<float4 *>(&leaves[i]);
 #pragma unroll
     for (int k = 0; k < 5; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
+
+    // the conservative stand-in (see DstLeafPre): mean plane, averaged half edges, their dual vectors
+    float cen[3], nrm[3], h1[3], h2[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        cen[a] = 0.25f * ((c[0][a] + c[1][a]) + (c[2][a] + c[3][a]));
+        nrm[a] = n0[a] - n1[a];   // the strip's second triangle winds the other way
+        h1[a] = 0.25f * ((c[1][a] - c[0][a]) + (c[3][a] - c[2][a]));   // half of the averaged edge A->B / C->D
+        h2[a] = 0.25f * ((c[2][a] - c[0][a]) + (c[3][a] - c[1][a]));   // half of the averaged edge A->C / B->D
+    }
+    const float nl = sqrtf(nrm[0] * nrm[0] + nrm[1] * nrm[1] + nrm[2] * nrm[2]);
+    float fu[3], fv[3], t1[3], t2[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) nrm[a] = nrm[a] / nl;
+    cross_f(h2, nrm, t1);    // perpendicular to h2 and the normal
+    cross_f(nrm, h1, t2);
+    const float d1 = h1[0] * t1[0] + h1[1] * t1[1] + h1[2] * t1[2];
+    const float d2 = h2[0] * t2[0] + h2[1] * t2[1] + h2[2] * t2[2];
+    float mfu = 0.f, lim0 = 0.f, dev = 0.f;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        fu[a] = t1[a] / d1;
+        fv[a] = t2[a] / d2;
+    }
+    mfu = fmaxf(sqrtf(fu[0] * fu[0] + fu[1] * fu[1] + fu[2] * fu[2]), sqrtf(fv[0] * fv[0] + fv[1] * fv[1] + fv[2] * fv[2]));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float w[3] = {c[k][0] - cen[0], c[k][1] - cen[1], c[k][2] - cen[2]};
+        lim0 = fmaxf(lim0, fabsf(fu[0] * w[0] + fu[1] * w[1] + fu[2] * w[2]));
+        lim0 = fmaxf(lim0, fabsf(fv[0] * w[0] + fv[1] * w[1] + fv[2] * w[2]));
+        dev = fmaxf(dev, fabsf(nrm[0] * w[0] + nrm[1] * w[1] + nrm[2] * w[2]));
+    }
+    // A ray that meets the quad at less than 0.05 rad-ish from its plane skips the stand-in (trace kernels), so a
+    // corner that is `dev` off the mean plane moves a hit by at most 20 dev along the plane; margins of 2.
+    float tdev = 40.0f * dev;
+    lim0 = lim0 * 1.002f + tdev * mfu;
+    const bool ok = isfinite(mfu) && isfinite(lim0) && isfinite(tdev) && isfinite(cen[0] + cen[1] + cen[2]) &&
+                    isfinite(nrm[0] + nrm[1] + nrm[2]) && nl > 0.f;
+    float pr[16];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        pr[a] = ok ? cen[a] : 0.f;
+        pr[3 + a] = ok ? nrm[a] : 0.f;
+        pr[6 + a] = ok ? fu[a] : 0.f;
+        pr[9 + a] = ok ? fv[a] : 0.f;
+    }
+    pr[12] = ok ? mfu : INFINITY;
+    pr[13] = ok ? lim0 : INFINITY;
+    pr[14] = ok ? tdev : INFINITY;
+    pr[15] = 0.f;
+    float4 *pdst = reinterpret_cast<float4 *>(&pre[i]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) pdst[k] = make_float4(pr[4 * k], pr[4 * k + 1], pr[4 * k + 2], pr[4 * k + 3]);
 }
 
 // Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes and goes on.
@@ -461,6 +515,8 @@ int ensure_capacity(dst_ctx *ctx, uint32_t P) {
     DST_HIP(ctx, hipMalloc((void **)&ctx->nodes, sizeof(DstNode) * std::max<size_t>(n - 1, 1)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->wide, sizeof(DstWideNode) * std::max<size_t>(n - 1, 1)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->leaves, sizeof(DstLeaf) * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->pre, sizeof(DstLeafPre) * (n + 1)));   // the trace kernels fetch them in pairs
+    DST_HIP(ctx, hipMemset(ctx->pre + n, 0, sizeof(DstLeafPre)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->node_parent, sizeof(uint32_t) * n));
     DST_HIP(ctx, hipMalloc((void **)&ctx->leaf_parent, sizeof(uint32_t) * n));
     DST_HIP(ctx, hipMalloc((void **)&ctx->flags, sizeof(uint32_t) * n));
@@ -510,6 +566,7 @@ void dst_lbvh_free(dst_ctx *ctx) {
     rel(ctx->nodes);
     rel(ctx->wide);
     rel(ctx->leaves);
+    rel(ctx->pre);
     rel(ctx->node_parent);
     rel(ctx->leaf_parent);
     rel(ctx->flags);
@@ -534,7 +591,8 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
         ctx->n_leaves = P;
     }
     if (fit_flags == nullptr) fit_flags = ctx->flags;   // after ensure_capacity: a first build allocates them there
-    if (fit_flags == nullptr || ctx->nodes == nullptr || ctx->leaves == nullptr || ctx->vals[0] == nullptr)
+    if (fit_flags == nullptr || ctx->nodes == nullptr || ctx->leaves == nullptr || ctx->pre == nullptr ||
+        ctx->vals[0] == nullptr)
         return dst_fail(ctx, DST_E_DEVICE, "acceleration structure buffers are not allocated");
     const uint32_t n = P;
     int4 *quad_ids = reinterpret_cast<int4 *>(ctx->quad_ids);
@@ -573,7 +631,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
         }
     }
     hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0], ctx->leaves,
-                       n);
+                       ctx->pre, n);
     hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, fit_flags, 0u, n);
     hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
                        fit_flags, ctx->leaves, n);

@@ -156,6 +156,7 @@ struct RaySlab {   // per-lane precomputation for the conservative slab test
     float ix, iy, iz;     // 1/d, with tiny components pushed away from zero
     float nx, ny, nz;     // -o * (1/d)
     float wx, wy, wz;     // interval widening per axis
+    float max_abs;        // largest vertex coordinate of the scene (uniform)
 };
 
 __device__ __forceinline__ float safe_inv(float d) {
@@ -175,6 +176,7 @@ __device__ __forceinline__ RaySlab make_slab(F3 o, F3 d, float max_abs) {
     // The quad test works in origin-relative fp32 coordinates, so it can accept a ray that passes
     // a few ulps of (|o| + |vertex|) outside the quad; boxes are widened by well above that.
     float oa = __builtin_fmaxf(__builtin_fabsf(o.x), __builtin_fmaxf(__builtin_fabsf(o.y), __builtin_fabsf(o.z)));
+    s.max_abs = max_abs;
     float pad = 4e-6f * (oa + max_abs);
     s.wx = pad * __builtin_fabsf(s.ix);
     s.wy = pad * __builtin_fabsf(s.iy);
@@ -234,19 +236,60 @@ __device__ __forceinline__ void kbuf_insert(KBuf &b, uint64_t x, bool on) {
 #ifdef DST_STATS
 struct WaveStats { unsigned long long nodes, leaves, t_trav, t_comp, chunks, leaf_any, t_plan, t_hb, steps; };
 #define STAT(x) x
+#define WSP , ws
 #else
 #define STAT(x)
+#define WSP
 #endif
 
-// Test all lanes' rays against one quad record and admit the hits into the lanes' buffers.
-__device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
+// Per-lane constants of the conservative stand-in for the quad test (DstLeafPre).  With S = |o|_max + the largest
+// vertex coordinate: the stand-in's distance along the ray is off by at most about 3.4e-5 S/|d| + 1e-5 |t| when
+// |n.d| >= 0.05 |d| (flatter rays skip the stand-in), its hit point by 7e-5 S; the margins below are twice that.
+struct RayPre {
+    float padw;     // in-plane slack, world units
+    float tp;       // slack on the distance along the ray
+    float graze;    // |n.d| below this: too flat for the stand-in
+    float inv_dl;   // 1 / |d|
+};
+__device__ __forceinline__ RayPre make_pre(F3 o, F3 d, float max_abs) {
+    RayPre r;
+    const float oa = __builtin_fmaxf(__builtin_fabsf(o.x), __builtin_fmaxf(__builtin_fabsf(o.y), __builtin_fabsf(o.z)));
+    const float S = oa + max_abs;
+    const float dl = __builtin_sqrtf(d.x * d.x + d.y * d.y + d.z * d.z);
+    r.inv_dl = 1.0f / dl;
+    r.padw = 1.5e-4f * S;
+    r.tp = 1e-4f * S * r.inv_dl;
+    r.graze = 0.05f * dl;
+    return r;
+}
+
+// The stand-in test of one quad for all lanes (about 28 instructions): false = this lane's ray cannot pass the exact test.
+__device__ __forceinline__ bool quad_may_hit(const uint32_t (&Q)[15], const RayPre &rp, F3 o, F3 d, bool active, float tmax) {
+#define QF(k) __uint_as_float(Q[k])
+    const float hx = QF(0) - o.x, hy = QF(1) - o.y, hz = QF(2) - o.z;
+    const float qd = __builtin_fmaf(QF(5), d.z, __builtin_fmaf(QF(4), d.y, QF(3) * d.x));
+    const float ph = __builtin_fmaf(QF(5), hz, __builtin_fmaf(QF(4), hy, QF(3) * hx));
+    const float t = ph * __builtin_amdgcn_rcpf(qd);
+    const float wx = __builtin_fmaf(t, d.x, -hx), wy = __builtin_fmaf(t, d.y, -hy), wz = __builtin_fmaf(t, d.z, -hz);
+    const float s = __builtin_fmaf(QF(8), wz, __builtin_fmaf(QF(7), wy, QF(6) * wx));
+    const float r = __builtin_fmaf(QF(11), wz, __builtin_fmaf(QF(10), wy, QF(9) * wx));
+    const float m = __builtin_fmaxf(__builtin_fabsf(s), __builtin_fabsf(r));
+    const float lim = __builtin_fmaf(rp.padw, QF(12), QF(13));
+    const float tpq = __builtin_fmaf(QF(14), rp.inv_dl, rp.tp);
+    // every comparison is written so that a NaN keeps the ray in
+    const bool flat = __builtin_fabsf(qd) < rp.graze;
+    const bool out = (m > lim) || (t < -tpq) || (__builtin_fmaf(t, 0.9999f, -tpq) > tmax);
+#undef QF
+    return active && (flat || !out);
+}
+
+// The exact test of one quad record for all lanes; hits are admitted into the lanes' buffers.
+__device__ __forceinline__ void quad_exact(const uint32_t (&L)[19], F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
 #ifdef DST_STATS
-                                          , WaveStats &ws
+                                           , WaveStats &ws
 #endif
 ) {
-    uint32_t L[19];
-    load_uniform<19>(leaf, L);
-    STAT(ws.leaves++;)
+    STAT(ws.t_plan++;)
 #define LF3(k) f3(__uint_as_float(L[k]), __uint_as_float(L[(k) + 1]), __uint_as_float(L[(k) + 2]))
     float t = 0.f;
     uint32_t tri = 0u;
@@ -261,6 +304,38 @@ __device__ __forceinline__ void test_leaf(const DstLeaf *leaf, F3 o, F3 d, bool 
     }
 }
 
+// A leaf group (up to DST_GROUP quads, consecutive records) against all lanes' rays.  The stand-in records of
+// two quads are fetched together, then the exact records of those that some lane's ray may hit, again together:
+// one trip to memory per stage instead of one per quad.
+__device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t first, uint32_t count, const RayPre &rp,
+                                           F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
+#ifdef DST_STATS
+                                           , WaveStats &ws
+#endif
+) {
+#pragma unroll 1
+    for (uint32_t q0 = 0; q0 < count; q0 += 2) {
+        const bool two = q0 + 1u < count;
+        // the record after the last quad of the structure exists (the array has one spare record)
+        uint32_t Q0[15], Q1[15];
+        load_uniform<15>(&acc.pre[first + q0], Q0);
+        load_uniform<15>(&acc.pre[first + q0 + 1u], Q1);
+        STAT(ws.leaves += two ? 2 : 1;)
+        const float tmax = kb_t(buf.e[kChunk - 1]);
+        const bool k0 = quad_may_hit(Q0, rp, o, d, active, tmax);
+        const bool k1 = quad_may_hit(Q1, rp, o, d, active && two, tmax);
+        uint32_t todo = (wave_ballot(k0) != 0ull ? 1u : 0u) | (wave_ballot(k1) != 0ull ? 2u : 0u);
+#pragma unroll 1
+        while (todo != 0u) {
+            const uint32_t k = (todo & 1u) ? 0u : 1u;
+            todo &= ~(1u << k);
+            uint32_t L[19];
+            load_uniform<19>(&acc.leaves[first + q0 + k], L);
+            quad_exact(L, o, d, active, buf, cnt WSP);
+        }
+    }
+}
+
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
 // to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow: nodes and quads
 // are fetched once per wave, the stack is two VGPRs addressed by lane (128 entries: the binary hierarchy
@@ -270,12 +345,10 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                                             bool active, int rep, KBuf &buf, uint32_t &cnt
 #ifdef DST_STATS
                                             , WaveStats &ws
-#define WSP , ws
-#else
-#define WSP
 #endif
 ) {
     const uint32_t lane = __lane_id();
+    const RayPre rp = make_pre(o, d, slab.max_abs);
     RaySlabFast fs;
     // byte offsets of the near / far face arrays inside a wide node (lox 0, loy 16, loz 32, hix 48, hiy 64, hiz 80)
     uint32_t onx = 0, ony = 16, onz = 32, ofx = 48, ofy = 64, ofz = 80;
@@ -293,8 +366,7 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
     for (uint32_t budget = 2u * acc.n_leaves + 8u; budget != 0u; --budget) {
         if (ref & DST_LEAF_BIT) {
             const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
-            for (uint32_t q = 0; q < count && first + q < acc.n_leaves; ++q)
-                test_leaf(&acc.leaves[first + q], o, d, active, buf, cnt WSP);
+            if (first + count <= acc.n_leaves) test_group(acc, first, count, rp, o, d, active, buf, cnt WSP);
         } else {
             if (ref + 1u >= acc.n_leaves) break;   // not a node of this hierarchy
             const char *node = reinterpret_cast<const char *>(&acc.wide[ref]);
@@ -1258,20 +1330,23 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         bid = (blockIdx.x >> 5) * 8u + (blockIdx.x & 7u);
         wv = (blockIdx.x >> 3) & 3u;
     }
-    // Blocks keep the dispatch order (row-major over the 16x16 pixel tiles).  Re-numbering them so that each of
-    // the 8 XCDs owns a band or whole rows of the image was measured and is slower on the 1080p room scene
-    // (+15 % / +8 % forward): the chip then works on 8 distant image regions at once and the shared last-level
-    // cache sees 8 times more distinct BVH data, which costs more than the per-XCD L2 gains.
+    // Blocks keep the dispatch order (row-major over the 16x16 pixel tiles).  Two re-numberings that give each of the
+    // 8 XCDs (workgroup number mod 8, an L2 each) its own part of the image were measured on the 1080p room scene
+    // and are slower: a band or whole rows per XCD (+15 % / +8 % forward: eight distant image regions in flight,
+    // eight times more distinct BVH data in the shared last-level cache), and compact neighbouring patches of 2x4
+    // to 8x16 blocks per XCD inside super-tiles (+1 % to +13 %, more with larger patches).
+    const uint32_t bx = bid % btiles_x, by = bid / btiles_x;
+    if (2u * by >= tiles_y) return;   // padding of the forward grid (whole blocks)
     RecView rv = {nullptr, nullptr, nullptr, 0u};
     if (REC) {
         const uint32_t n_waves = btiles_x * ((tiles_y + 1u) / 2u) * kWavesPerBlock, slots_ = (uint32_t)p.mtd_alloc + 1u;
         const uint64_t dir_words = ((uint64_t)n_waves * slots_ + 1u) / 2u;
         rv.base = p.hit_record;
-        rv.dir = reinterpret_cast<uint32_t *>(p.hit_record + 2) + (size_t)(bid * kWavesPerBlock + wv) * slots_;
+        rv.dir = reinterpret_cast<uint32_t *>(p.hit_record + 2) + (size_t)((by * btiles_x + bx) * kWavesPerBlock + wv) * slots_;
         rv.blocks = p.hit_record + 2 + dir_words;
         rv.capacity = p.hit_record_blocks;
     }
-    const uint32_t ty = 2u * (bid / btiles_x) + (wv >> 1), tx = 2u * (bid % btiles_x) + (wv & 1u);
+    const uint32_t ty = 2u * by + (wv >> 1), tx = 2u * bx + (wv & 1u);
     const bool wave_on = ty < tiles_y && tx < tiles_x;
     if (!BWD && !wave_on) return;   // the backward kernel keeps every wave for the block-wide flush below
     const uint32_t lane = threadIdx.x % DST_WAVE;
@@ -1372,6 +1447,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                 atomicAdd(p.counters + 5, ws.t_comp);
                 atomicAdd(p.counters + 6, ws.chunks);
                 atomicAdd(p.counters + 7, ws.leaf_any);
+                atomicAdd(p.counters + 8, ws.t_plan);   // exact quad tests run (forward only)
 #endif
             }
         }
@@ -1508,9 +1584,10 @@ TileGrid tile_grid(int H, int W) {
 
 template <bool BWD, bool REC>
 void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipStream_t stream) {
-    dim3 grid(t.btiles_x * t.btiles_y), block(kWavesPerBlock * DST_WAVE);
+    const uint32_t n_blocks = t.btiles_x * t.btiles_y;
+    dim3 grid(n_blocks), block(kWavesPerBlock * DST_WAVE);
     if (!BWD && kFwdWavesPerBlock == 1) {
-        grid = dim3((t.btiles_x * t.btiles_y + 7u) / 8u * 32u);
+        grid = dim3((n_blocks + 7u) / 8u * 32u);
         block = dim3(DST_WAVE);
     }
     // The per-lane walk is built into the kernels used where waves of unrelated rays are to be expected:
@@ -1561,6 +1638,7 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     DstAccelView acc;
     acc.wide = ctx->wide;
     acc.leaves = ctx->leaves;
+    acc.pre = ctx->pre;
     acc.bounds = ctx->bounds;
     acc.n_leaves = ctx->n_leaves;
     acc.root = dst_root_ref(ctx->n_leaves);
