@@ -108,6 +108,23 @@ def main():
     build_ms = sorted(timed_build(True) for _ in range(5))[2]
     refit_ms = sorted(timed_build(False) for _ in range(5))[2]
 
+    # a dynamic frame's geometry update, two ways: the reference's (tensor operations make the quads, then a refit
+    # from them) and this library's extension (one kernel makes the quads and refits)
+    def timed(fn):
+        a, b = ev(), ev()
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b)
+    timed(lambda: S.get_triangles(g["means3D"], g["scales"], g["rotations"]))
+    quads_ms = sorted(timed(lambda: S.get_triangles(g["means3D"], g["scales"], g["rotations"])) for _ in range(5))[2]
+    v_out = torch.empty_like(g["vertices"])
+    fused = lambda: tracer.refit_from_surfels(g["means3D"], g["scales"], g["rotations"], v_out)  # noqa: E731
+    timed(fused)
+    refit_fused_ms = sorted(timed(fused) for _ in range(5))[2]
+    tracer.build_acceleration_structure(g["vertices"], g["faces"], False)   # back to the scene's own quads
+
     e = torch.empty(0, device=dev)
     bg = torch.zeros(3, device=dev)
     eye = torch.eye(4, device=dev)
@@ -183,6 +200,7 @@ def main():
                    "aux_channels": aux, "training": True, "seed": 0},
         "fwd_kernel_ms": round(fwd_ms, 4), "bwd_kernel_ms": round(bwd_ms, 4),
         "bvh_build_ms": round(build_ms, 4), "bvh_refit_ms": round(refit_ms, 4),
+        "quads_by_tensor_ops_ms": round(quads_ms, 4), "bvh_refit_from_surfels_ms": round(refit_fused_ms, 4),
         "hits_evaluated_per_ray": round(n_proc / R, 3), "hits_composited_per_ray": round(n_con / R, 3),
         "algorithmic_bytes": int(A_total), "hbm_peak_frac": round(A_total / (ms_per_step * 1e-3) / (HBM_PEAK_GBS * 1e9), 5),
         "roofline": roofline, "roofline_kernels": per_kernel,

@@ -111,6 +111,22 @@ int dst_refit_accel_static(dst_ctx *ctx, const float *vertices, uint32_t n_verti
     return dst_lbvh_build(ctx, vertices, n_vertices, nullptr, ctx->n_leaves, false, (hipStream_t)stream, scratch);
 }
 
+int dst_refit_from_surfels(dst_ctx *ctx, const float *means3D, const float *scales, const float *rotations,
+                           uint32_t n_surfels, float *vertices_out, void *stream) {
+    if (!ctx) return DST_E_INVALID;
+    if (!means3D || !scales || !rotations)
+        return dst_fail(ctx, DST_E_INVALID, "means3D, scales and rotations are required");
+    if (!ctx->built) return dst_fail(ctx, DST_E_NO_ACCEL, "refit before any build");
+    if (n_surfels != ctx->n_leaves)
+        return dst_fail(ctx, DST_E_TOPOLOGY, "refit with a different number of surfels");
+    if (!ctx->canonical)
+        return dst_fail(ctx, DST_E_TOPOLOGY,
+                        "refit from surfel parameters needs a structure built from quads in rows 4g..4g+3 of the "
+                        "vertex buffer (triangles [4g,4g+1,4g+2],[4g+1,4g+2,4g+3])");
+    const DstSurfelSource src = {means3D, scales, rotations, vertices_out};
+    return dst_lbvh_build(ctx, nullptr, 0, nullptr, n_surfels, false, (hipStream_t)stream, nullptr, &src);
+}
+
 int dst_trace_forward(dst_ctx *ctx, const DstParams *p, void *stream) {
     if (!ctx) return DST_E_INVALID;
     int rc = check_common(ctx, p);

@@ -88,6 +88,7 @@ struct dst_ctx {
     uint32_t capacity = 0;      // surfels the buffers can hold
     bool built = false;
     uint32_t built_vertices = 0;   // rows of the vertex buffer the stored quad ids were validated against
+    bool canonical = false;        // the build's quads were rows 4g..4g+3 of the vertex buffer, in that order
     uint32_t builds = 0, refits = 0;
     DstNode *nodes = nullptr;
     DstWideNode *wide = nullptr;
@@ -111,9 +112,16 @@ static inline uint32_t dst_root_ref(uint32_t n_leaves) {
 }
 
 // lbvh.hip
+// Refit source other than a vertex buffer: the surfel parameters themselves (device pointers).
+struct DstSurfelSource {
+    const float *means, *scales, *rotations;   // (P,3) (P,2) (P,4)
+    float *vertices_out;                        // (4P,3) or nullptr
+};
 // `fit_flags`: arrival counters of the bottom-up fit (one per surfel); nullptr = the context's own.
+// `surfels`: refit only; the quads are generated from the surfel parameters instead of read from `vertices`.
 int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
-                   uint32_t n_surfels, bool rebuild, hipStream_t stream, uint32_t *fit_flags = nullptr);
+                   uint32_t n_surfels, bool rebuild, hipStream_t stream, uint32_t *fit_flags = nullptr,
+                   const DstSurfelSource *surfels = nullptr);
 // Per-device address of the static scratch array (set up once per device by dst_create).
 int dst_static_scratch_init(dst_ctx *ctx);
 uint32_t *dst_static_scratch(const dst_ctx *ctx);

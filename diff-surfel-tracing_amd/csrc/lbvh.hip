@@ -74,6 +74,8 @@ __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vert
             if (bad) {
                 atomicOr(&bounds->bad_topology, 1u);
                 q = make_int4(0, 0, 0, 0);
+            } else if (q.x != (int)(4u * g) || q.y != q.x + 1 || q.z != q.x + 2 || q.w != q.x + 3) {
+                atomicOr(&bounds->bad_topology, 2u);   // valid, but not rows 4g..4g+3 in order
             }
             quad_ids[g] = q;
         } else {
@@ -291,24 +293,10 @@ __global__ void k_karras(const uint32_t *__restrict__ keys, DstNode *__restrict_
     if (i == 0) node_parent[0] = DST_NO_PARENT;
 }
 
-// Leaf records in Morton order (also the whole of a refit's geometry update).  The plane normals use the
-// fused form the hit test is defined with: cross(x,y).x = fma(x.y, y.z, -(x.z*y.y)), and so on.
-__global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
-                            const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
-                            DstLeafPre *__restrict__ pre, uint32_t n) {
-    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    uint32_t g = sorted_ids[i];
-    int4 q = quad_ids[g];
-    const int ids[4] = {q.x, q.y, q.z, q.w};
-    float c[4][3];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const float *v = vertices + (size_t)ids[k] * 3;
-        c[k][0] = v[0];
-        c[k][1] = v[1];
-        c[k][2] = v[2];
-    }
+// Leaf record + conservative stand-in of one quad (corners c[0..3] = A,B,C,D, surfel id g) at leaf position i.
+// The plane normals use the fused form the hit test is defined with: cross(x,y).x = fma(x.y, y.z, -(x.z*y.y)), ...
+__device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, uint32_t i, DstLeaf *__restrict__ leaves,
+                                           DstLeafPre *__restrict__ pre) {
     auto cross_f = [](const float *x, const float *y, float *out) {
         out[0] = __builtin_fmaf(x[1], y[2], -(x[2] * y[1]));
         out[1] = __builtin_fmaf(x[2], y[0], -(x[0] * y[2]));
@@ -391,6 +379,70 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
     float4 *pdst = reinterpret_cast<float4 *>(&pre[i]);
 #pragma unroll
     for (int k = 0; k < 4; ++k) pdst[k] = make_float4(pr[4 * k], pr[4 * k + 1], pr[4 * k + 2], pr[4 * k + 3]);
+}
+
+// Leaf records in Morton order (also the whole of a refit's geometry update).
+__global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
+                            const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
+                            DstLeafPre *__restrict__ pre, uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t g = sorted_ids[i];
+    int4 q = quad_ids[g];
+    const int ids[4] = {q.x, q.y, q.z, q.w};
+    float c[4][3];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float *v = vertices + (size_t)ids[k] * 3;
+        c[k][0] = v[0];
+        c[k][1] = v[1];
+        c[k][2] = v[2];
+    }
+    write_leaf(c, g, i, leaves, pre);
+}
+
+// The same for a refit straight from the surfel parameters: the four corners of surfel g are
+//   v_k = (mean + a_k * (sx * R[:,0])) + b_k * (sy * R[:,1]),  (a,b) = (-3,3), (-3,-3), (3,3), (3,-3),
+// R the rotation of the quaternion (w,x,y,z) divided by its norm sqrt(((w*w + x*x) + y*y) + z*z): the quads of
+// the 2DGS convention (reference example/utils/gaussian_utils.py:176-210), every operation in fp32, rounded once,
+// in exactly this order (this file is compiled without contraction).  Optionally writes the corners to
+// `vertices_out` (4P,3) in the canonical order (rows 4g..4g+3) for the trace calls, and reduces the largest
+// |coordinate| the trace kernels size their padding with.
+__global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const float *__restrict__ scales,
+                                         const float *__restrict__ rotations, const uint32_t *__restrict__ sorted_ids,
+                                         DstLeaf *__restrict__ leaves, DstLeafPre *__restrict__ pre,
+                                         float *__restrict__ vertices_out, DstBounds *__restrict__ bounds, uint32_t n) {
+    float mabs = 0.f;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        const uint32_t g = sorted_ids[i];
+        const float q0 = rotations[4 * (size_t)g], q1 = rotations[4 * (size_t)g + 1], q2 = rotations[4 * (size_t)g + 2],
+                    q3 = rotations[4 * (size_t)g + 3];
+        const float nrm = sqrtf(((q0 * q0 + q1 * q1) + q2 * q2) + q3 * q3);
+        const float w = q0 / nrm, x = q1 / nrm, y = q2 / nrm, z = q3 / nrm;
+        const float sx = scales[2 * (size_t)g], sy = scales[2 * (size_t)g + 1];
+        const float u[3] = {(1.f - 2.f * (y * y + z * z)) * sx, (2.f * (x * y + w * z)) * sx, (2.f * (x * z - w * y)) * sx};
+        const float v[3] = {(2.f * (x * y - w * z)) * sy, (1.f - 2.f * (x * x + z * z)) * sy, (2.f * (y * z + w * x)) * sy};
+        const float m[3] = {means[3 * (size_t)g], means[3 * (size_t)g + 1], means[3 * (size_t)g + 2]};
+        const float sa[4] = {-3.f, -3.f, 3.f, 3.f}, sb[4] = {3.f, -3.f, 3.f, -3.f};
+        float c[4][3];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                c[k][a] = (m[a] + sa[k] * u[a]) + sb[k] * v[a];
+                mabs = fmaxf(mabs, fabsf(c[k][a]));
+            }
+        if (vertices_out != nullptr) {
+            float4 *dst = reinterpret_cast<float4 *>(vertices_out + 12 * (size_t)g);   // 48 bytes per surfel
+            dst[0] = make_float4(c[0][0], c[0][1], c[0][2], c[1][0]);
+            dst[1] = make_float4(c[1][1], c[1][2], c[2][0], c[2][1]);
+            dst[2] = make_float4(c[2][2], c[3][0], c[3][1], c[3][2]);
+        }
+        write_leaf(c, g, i, leaves, pre);
+    }
+    mabs = wave_max(mabs);
+    if ((threadIdx.x & (DST_WAVE - 1)) == 0 && mabs > 0.f && mabs < INFINITY)
+        atomicMax(&bounds->max_abs, __float_as_uint(mabs));
 }
 
 // Bottom-up fit: each leaf climbs; the second thread to reach a node merges the two child boxes and goes on.
@@ -583,7 +635,7 @@ void dst_lbvh_free(dst_ctx *ctx) {
 }
 
 int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles, uint32_t P,
-                   bool rebuild, hipStream_t stream, uint32_t *fit_flags) {
+                   bool rebuild, hipStream_t stream, uint32_t *fit_flags, const DstSurfelSource *surfels) {
     if (rebuild) {
         ctx->built = false;
         int rc = ensure_capacity(ctx, P);
@@ -600,7 +652,11 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
 
     hipLaunchKernelGGL(k_init_bounds, dim3(1), dim3(64), 0, stream, ctx->bounds);
     const dim3 setup_grid(std::min<uint32_t>(grid_for(n).x, 1024u));   // 4 blocks per CU, each thread takes several surfels
-    if (rebuild)
+    if (surfels != nullptr) {
+        // refit from the surfel parameters: corners, leaf records and the coordinate bound in one kernel
+        hipLaunchKernelGGL(k_leaf_fill_from_surfels, setup_grid, dim3(kBlock), 0, stream, surfels->means, surfels->scales,
+                           surfels->rotations, ctx->vals[0], ctx->leaves, ctx->pre, surfels->vertices_out, ctx->bounds, n);
+    } else if (rebuild)
         hipLaunchKernelGGL(k_quad_setup<true>, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
                            quad_ids, centroids, ctx->bounds, n);
     else
@@ -630,8 +686,9 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
             hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(kBlock), 0, stream, ctx->leaf_parent, DST_NO_PARENT, 1u);
         }
     }
-    hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0], ctx->leaves,
-                       ctx->pre, n);
+    if (surfels == nullptr)
+        hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0],
+                           ctx->leaves, ctx->pre, n);
     hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, fit_flags, 0u, n);
     hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
                        fit_flags, ctx->leaves, n);
@@ -642,7 +699,8 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     if (rebuild) {
         DST_HIP(ctx, hipMemcpyAsync(ctx->bounds_host, ctx->bounds, sizeof(DstBounds), hipMemcpyDeviceToHost, stream));
         DST_HIP(ctx, hipStreamSynchronize(stream));
-        if (ctx->bounds_host->bad_topology)
+        ctx->canonical = (ctx->bounds_host->bad_topology & 2u) == 0u;
+        if (ctx->bounds_host->bad_topology & 1u)
             return dst_fail(ctx, DST_E_TOPOLOGY,
                             "triangles must come in pairs [a,b,c],[b,c,d] per surfel with ids inside vertices");
         for (int a = 0; a < 3; ++a) {

@@ -143,6 +143,9 @@ __device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 B, F3 C, F3 Dv, F3
     return (t > 0.0f) && (t < kInfDepth);
 }
 
+// v_writelane_b32: value (uniform) into lane `lane` (uniform) of `old`; the compiler offers no builtin for it.
+__device__ int dst_writelane(int value, int lane, int old) __asm("llvm.amdgcn.writelane.i32");
+
 // ---- wave-uniform fetches ---------------------------------------------------------------------------------
 typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
 template <int N>
@@ -263,8 +266,9 @@ __device__ __forceinline__ RayPre make_pre(F3 o, F3 d, float max_abs) {
     return r;
 }
 
-// The stand-in test of one quad for all lanes (about 28 instructions): false = this lane's ray cannot pass the exact test.
-__device__ __forceinline__ bool quad_may_hit(const uint32_t (&Q)[15], const RayPre &rp, F3 o, F3 d, bool active, float tmax) {
+// The stand-in test of one quad for all lanes (about 28 instructions), as a lane mask: bit clear = that lane's ray
+// cannot pass the exact test (lanes that are switched off come back set or clear; the caller masks them).
+__device__ __forceinline__ uint64_t quad_may_hit(const uint32_t (&Q)[16], const RayPre &rp, F3 o, F3 d, float tmax) {
 #define QF(k) __uint_as_float(Q[k])
     const float hx = QF(0) - o.x, hy = QF(1) - o.y, hz = QF(2) - o.z;
     const float qd = __builtin_fmaf(QF(5), d.z, __builtin_fmaf(QF(4), d.y, QF(3) * d.x));
@@ -276,11 +280,11 @@ __device__ __forceinline__ bool quad_may_hit(const uint32_t (&Q)[15], const RayP
     const float m = __builtin_fmaxf(__builtin_fabsf(s), __builtin_fabsf(r));
     const float lim = __builtin_fmaf(rp.padw, QF(12), QF(13));
     const float tpq = __builtin_fmaf(QF(14), rp.inv_dl, rp.tp);
-    // every comparison is written so that a NaN keeps the ray in
-    const bool flat = __builtin_fabsf(qd) < rp.graze;
-    const bool out = (m > lim) || (t < -tpq) || (__builtin_fmaf(t, 0.9999f, -tpq) > tmax);
+    // every comparison is written so that a NaN keeps the ray in; the lane masks are combined without branches
+    const uint64_t flat = wave_ballot(__builtin_fabsf(qd) < rp.graze);
+    const uint64_t out = wave_ballot(m > lim) | wave_ballot(t < -tpq) | wave_ballot(__builtin_fmaf(t, 0.9999f, -tpq) > tmax);
 #undef QF
-    return active && (flat || !out);
+    return flat | ~out;
 }
 
 // The exact test of one quad record for all lanes; hits are admitted into the lanes' buffers.
@@ -317,14 +321,15 @@ __device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t fir
     for (uint32_t q0 = 0; q0 < count; q0 += 2) {
         const bool two = q0 + 1u < count;
         // the record after the last quad of the structure exists (the array has one spare record)
-        uint32_t Q0[15], Q1[15];
-        load_uniform<15>(&acc.pre[first + q0], Q0);
-        load_uniform<15>(&acc.pre[first + q0 + 1u], Q1);
+        uint32_t Q0[16], Q1[16];
+        load_uniform<16>(&acc.pre[first + q0], Q0);
+        load_uniform<16>(&acc.pre[first + q0 + 1u], Q1);
         STAT(ws.leaves += two ? 2 : 1;)
         const float tmax = kb_t(buf.e[kChunk - 1]);
-        const bool k0 = quad_may_hit(Q0, rp, o, d, active, tmax);
-        const bool k1 = quad_may_hit(Q1, rp, o, d, active && two, tmax);
-        uint32_t todo = (wave_ballot(k0) != 0ull ? 1u : 0u) | (wave_ballot(k1) != 0ull ? 2u : 0u);
+        const uint64_t live = wave_ballot(active);
+        const uint64_t k0 = quad_may_hit(Q0, rp, o, d, tmax) & live;
+        const uint64_t k1 = two ? (quad_may_hit(Q1, rp, o, d, tmax) & live) : 0ull;
+        uint32_t todo = (k0 != 0ull ? 1u : 0u) | (k1 != 0ull ? 2u : 0u);
 #pragma unroll 1
         while (todo != 0u) {
             const uint32_t k = (todo & 1u) ? 0u : 1u;
@@ -374,12 +379,14 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
             const float tmax = active ? kb_t(buf.e[kChunk - 1]) : -1.0f;
             uint32_t tail[5];
             load_uniform<5>(node + 96, tail);      // ref[4], count
-            const uint32_t n_child = tail[4];
             uint32_t hit = 0u;                     // bit k: some lane enters child k
             {
                 uint32_t NX[4], NY[4], NZ[4], FX[4], FY[4], FZ[4];
                 load_uniform<4>(node + onx, NX); load_uniform<4>(node + ony, NY); load_uniform<4>(node + onz, NZ);
                 load_uniform<4>(node + ofx, FX); load_uniform<4>(node + ofy, FY); load_uniform<4>(node + ofz, FZ);
+                // one trip to memory per node: without this the compiler fetches the references and the count only
+                // when they are used, two more waits behind the first
+                asm volatile("" ::"s"(tail[0]), "s"(tail[1]), "s"(tail[2]), "s"(tail[3]), "s"(tail[4]), "s"(NX[0]));
 #pragma unroll
                 for (int k = 0; k < DST_WIDE; ++k) {
                     float tn;
@@ -388,19 +395,17 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                                                      __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn);
                     hit |= (h != 0ull) ? (1u << k) : 0u;
                 }
-                hit &= (1u << n_child) - 1u;       // unused slots are never entered
+                hit &= (1u << tail[4]) - 1u;       // unused slots are never entered
             }
             if (hit != 0u) {
                 // Children are taken in stored order: the first one that is hit next, the others deferred (last
                 // first).  Ordering them by entry distance was measured: 3 % fewer visits, but the scalar work of
                 // the sort costs more than those visits.
-#define DST_PUSH(v)                                                                   \
-    {   /* no lane has the number 255: the register that is not meant keeps its content */ \
-        const uint32_t slot = (uint32_t)sp & 63u;                                     \
-        const uint32_t t0 = sp < 64 ? slot : 255u, t1 = sp < 64 ? 255u : slot;        \
-        stack0 = (lane == t0) ? (v) : stack0;                                         \
-        stack1 = (lane == t1) ? (v) : stack1;                                         \
-        sp = min(sp + 1, 2 * DST_WAVE - 1);                                           \
+#define DST_PUSH(v)                                                                                          \
+    {                                                                                                        \
+        if (sp < 64) stack0 = (uint32_t)dst_writelane((int)(v), sp, (int)stack0);               \
+        else stack1 = (uint32_t)dst_writelane((int)(v), sp - 64, (int)stack1);                  \
+        sp = min(sp + 1, 2 * DST_WAVE - 1);                                                                  \
     }
                 if ((hit & 8u) && (hit & 7u)) DST_PUSH(tail[3])
                 if ((hit & 4u) && (hit & 3u)) DST_PUSH(tail[2])
@@ -1130,6 +1135,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         for (int it = 0; it < kChunk; ++it) {
             const bool on = live && !stop && (uint32_t)it < cnt;
             if (wave_ballot(on) == 0ull) break;
+            STAT(if (!BWD) { ws.steps++; ws.t_hb += __popcll(wave_ballot(on)); })
             // next entry in depth order (consumed slots need no reset: the buffer is rebuilt for every chunk)
             uint64_t e;
             Ahead cur = nx;
@@ -1448,6 +1454,8 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                 atomicAdd(p.counters + 6, ws.chunks);
                 atomicAdd(p.counters + 7, ws.leaf_any);
                 atomicAdd(p.counters + 8, ws.t_plan);   // exact quad tests run (forward only)
+                atomicAdd(p.counters + 9, ws.steps);    // compositing iterations of the wave
+                atomicAdd(p.counters + 10, ws.t_hb);    // lanes with an entry, summed over those iterations
 #endif
             }
         }

@@ -45,7 +45,7 @@ class DstAccelInfo(C.Structure):
 
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
            "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params",
-           "dst_hit_record_layout", "dst_refit_accel_static")
+           "dst_hit_record_layout", "dst_refit_accel_static", "dst_refit_from_surfels")
 
 _lib = None
 
@@ -65,6 +65,8 @@ def load_library():
     L.dst_destroy.argtypes = [C.c_void_p]
     L.dst_build_accel.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_int, C.c_void_p]
     L.dst_refit_accel_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p]
+    L.dst_refit_from_surfels.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p,
+                                         C.c_void_p]
     L.dst_trace_forward.argtypes = [C.c_void_p, C.POINTER(DstParams), C.c_void_p]
     L.dst_trace_backward.argtypes = [C.c_void_p, C.POINTER(DstParams), C.c_void_p]
     L.dst_last_error.restype = C.c_char_p
@@ -265,6 +267,26 @@ def build_acceleration_structure(ctx, vertices, triangles, rebuild):
                                         int(bool(rebuild)), _stream())
     _check(ctx, rc)
     ctx.num_surfels = f.size(0) // 2
+
+
+def refit_from_surfels(ctx, means3D, scales, rotations, vertices_out=None):
+    """Refit the structure straight from the surfel parameters (dst_refit_from_surfels in include/dst_api.h) and
+    return the quad corners (4P,3) the trace calls take as `vertices`, written by the same kernel.  No counterpart
+    in the reference, whose callers regenerate the quads with tensor operations and then call
+    build_acceleration_structure(v, f, rebuild=False)."""
+    m, s, q = _cuda_f32(means3D, "means3D"), _cuda_f32(scales, "scales"), _cuda_f32(rotations, "rotations")
+    P = m.size(0)
+    if m.dim() != 2 or m.size(1) != 3 or tuple(s.shape) != (P, 2) or tuple(q.shape) != (P, 4):
+        raise RuntimeError("means3D (P,3), scales (P,2) and rotations (P,4) are required")
+    if vertices_out is None:
+        vertices_out = torch.empty((4 * P, 3), dtype=torch.float32, device=m.device)
+    elif (not vertices_out.is_cuda or vertices_out.dtype != torch.float32 or not vertices_out.is_contiguous()
+          or vertices_out.numel() != 12 * P):
+        raise RuntimeError("vertices_out must be a contiguous CUDA float32 tensor of shape (4P,3)")
+    rc = load_library().dst_refit_from_surfels(ctx.handle, m.data_ptr(), s.data_ptr(), q.data_ptr(), P,
+                                               vertices_out.data_ptr(), _stream())
+    _check(ctx, rc)
+    return vertices_out
 
 
 def _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp, others_precomp,

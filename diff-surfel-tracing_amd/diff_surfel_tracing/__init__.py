@@ -141,6 +141,14 @@ class SurfelTracer(nn.Module):
         """Build (`rebuild` true) or refit in place the BVH over the surfel quads `vertices` (4P,3), `triangles` (2P,3)."""
         return _C.build_acceleration_structure(self.optix_context, vertices, triangles, rebuild)
 
+    def refit_from_surfels(self, means3D: torch.Tensor, scales: torch.Tensor, rotations: torch.Tensor,
+                           vertices_out: torch.Tensor = None) -> torch.Tensor:
+        """Extension (not in the reference): refit the BVH in place from the surfel parameters and return the quad
+        corners (4P,3) to pass to forward() as `vertices`: what `get_triangles` + `build_acceleration_structure(v, f,
+        rebuild=False)` do, in one kernel.  Needs a structure built from `get_triangles`-style quads."""
+        return _C.refit_from_surfels(self.optix_context, means3D.detach(), scales.detach(), rotations.detach(),
+                                     vertices_out)
+
     def forward(self, ray_o: torch.Tensor, ray_d: torch.Tensor, vertices: torch.Tensor, means3D: torch.Tensor,
                 grads3D: torch.Tensor, shs: torch.Tensor = None, colors_precomp: torch.Tensor = None,
                 others_precomp: torch.Tensor = None, opacities: torch.Tensor = None, scales: torch.Tensor = None,

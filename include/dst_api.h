@@ -130,6 +130,18 @@ void dst_destroy(dst_ctx *ctx);
 int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
                     uint32_t n_triangles, int rebuild, void *stream);
 
+/* Refit straight from the surfel parameters (no counterpart in the reference, where the caller regenerates the
+ * quads with tensor operations every frame: example/utils/gaussian_utils.py:176-210): the kernel that fills the
+ * leaf records builds the four corners of every surfel itself,
+ *     v_k = (mean + a_k * (sx * R[:,0])) + b_k * (sy * R[:,1]),   (a,b) = (-3,3), (-3,-3), (3,3), (3,-3),
+ * R = rotation of the quaternion (w,x,y,z) divided by its norm sqrt(((w*w + x*x) + y*y) + z*z), every operation
+ * in fp32, rounded once, in this order.  means3D (P,3), scales (P,2), rotations (P,4) are device pointers;
+ * vertices_out, if not NULL, receives the corners as a (4P,3) buffer in the order the trace calls expect
+ * (`vertices` of DstParams).  The structure must come from a build whose quads were rows 4g..4g+3 of its vertex
+ * buffer (what get_triangles produces), else DST_E_TOPOLOGY.  Stream-ordered, no wait. */
+int dst_refit_from_surfels(dst_ctx *ctx, const float *means3D, const float *scales, const float *rotations,
+                           uint32_t n_surfels, float *vertices_out, void *stream);
+
 /* Refit that allocates nothing: dst_build_accel with rebuild == 0, except that the scratch of the refit
  * kernels (one arrival counter per surfel for the bottom-up box fit) is a fixed array inside the library,
  * 4 bytes x DST_STATIC_REFIT_MAX_SURFELS = 8 MiB, which every GPU the library runs on holds until the process
