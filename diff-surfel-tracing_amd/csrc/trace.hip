@@ -609,6 +609,25 @@ template <int AUXM> struct RowLayout {
     static constexpr int rows_log2 = AUXM <= 2 ? DST_TABLE_ROWS_LOG2 : DST_TABLE_ROWS_LOG2 - 1;
     static constexpr int rows = 1 << rows_log2;
 };
+// The deterministic mode keeps 64-bit fixed-point sums in the table: half as many rows in the same memory.
+template <int AUXM, bool DET> struct TableRows {
+    static constexpr int rows_log2 = RowLayout<AUXM>::rows_log2 - (DET ? 1 : 0);
+    static constexpr int rows = 1 << rows_log2;
+};
+
+// ---- deterministic mode: sums in 64-bit fixed point ------------------------------------------------------
+// Integer addition is exact, so a sum of fixed-point numbers does not depend on the order of its terms: every
+// atomically accumulated value (LDS table, global memory) is converted first.  2^-36 units for the geometric
+// columns (scale, rotation, mean, densification: range +-6.7e7), 2^-40 for the others and for the blending
+// weights (+-4.2e6); a value outside the range saturates.
+constexpr int kDetShiftGeo = 36, kDetShiftOther = 40;
+__device__ __forceinline__ int det_shift(int col) { return (col >= kColScale && col < kColAux) ? kDetShiftGeo : kDetShiftOther; }
+__device__ __forceinline__ long long to_fixed(float v, int shift) {
+    float x = __builtin_ldexpf(v, shift);                       // exact scaling
+    x = __builtin_fminf(__builtin_fmaxf(x, -4.6e18f), 4.6e18f);   // |x| < 2^62; NaN becomes a bound
+    return (long long)x;
+}
+__device__ __forceinline__ float from_fixed(long long q, int shift) { return (float)__builtin_ldexp((double)q, -shift); }
 
 // Address in the caller's gradient tensors of column `col` of surfel g (nullptr: nothing to write).
 template <int AUXM>
@@ -644,7 +663,11 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
 // base[key] += v for every lane with `on`, wave-uniform call.  Neighbouring rays mostly composite the same surfel
 // in the same step, and atomics of one instruction to one address are served one after the other, so the lanes
 // of the most frequent keys are summed across the wave and their first lane adds the total.
-__device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t key, float v) {
+__device__ __forceinline__ void wave_add_grouped(float *base, unsigned long long *det, bool on, uint32_t key, float v) {
+    auto add = [&](uint32_t k, float x) {
+        if (det != nullptr) atomicAdd(det + k, (unsigned long long)to_fixed(x, kDetShiftOther));
+        else aadd(base + k, x);
+    };
     const uint32_t lane = __lane_id();
     uint64_t rem = wave_ballot(on);
 #pragma unroll 1
@@ -655,12 +678,12 @@ __device__ __forceinline__ void wave_add_grouped(float *base, bool on, uint32_t 
         const uint64_t grp = wave_ballot(same);
         if (__popcll(grp) >= 3) {
             const float s = wave_sum_f32(same ? v : 0.f);
-            if (lane == (uint32_t)first) aadd(base + k0, s);
+            if (lane == (uint32_t)first) add(k0, s);
             on = on && !same;
         }
         rem &= ~grp;
     }
-    if (on) aadd(base + key, v);
+    if (on) add(key, v);
 }
 
 // Find or claim the table row of surfel g; -1 if none is free within a few probes.  keys[rows] counts the
@@ -697,7 +720,7 @@ constexpr int kStageCols = 16;                 // columns per tile
 constexpr int kStageStride = DST_WAVE + 1;     // floats per staged column: conflict-free writes and reads
 constexpr int kStageWords = kStageCols * kStageStride;
 typedef float v4f __attribute__((ext_vector_type(4)));
-template <int AUXM>
+template <int AUXM, bool DET>
 struct GradSink {
     const DstParams *p;
     float *rows;         // the block's table
@@ -738,13 +761,20 @@ struct GradSink {
         stray = did && !grouped;
         any_stray = wave_ballot(stray) != 0ull;
         out_on = (lane & 15u) < (uint32_t)n_groups;
-        own_slot = did ? table_slot<RowLayout<AUXM>::rows_log2>(keys, g) : -1;
+        own_slot = did ? table_slot<TableRows<AUXM, DET>::rows_log2>(keys, g) : -1;
         out_slot = __builtin_amdgcn_ds_bpermute((int)(leader << 2), own_slot);
         out_g = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader << 2), (int)g);
     }
 
     __device__ __forceinline__ void put(int slot, uint32_t surfel, int col, float v) const {
-        if (slot >= 0) {
+        if (DET) {
+            const long long q = to_fixed(v, det_shift(col));
+            if (slot >= 0)
+                __hip_atomic_fetch_add(reinterpret_cast<long long *>(rows) + (size_t)slot * RowLayout<AUXM>::stride + col, q,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            else if (grad_address<AUXM>(*p, surfel, col) != nullptr)
+                atomicAdd(p->det_workspace + (size_t)surfel * RowLayout<AUXM>::cols + col, (unsigned long long)q);
+        } else if (slot >= 0) {
             __hip_atomic_fetch_add(rows + (size_t)slot * RowLayout<AUXM>::stride + col, v, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_WORKGROUP);
         } else {
@@ -829,14 +859,14 @@ __device__ __forceinline__ F3 sh_direction_gradient(int deg, const float *__rest
 
 // Gradient of one composited hit (reference backward.cu:528-640 and 201-287, 68-166).
 // Pure gradient algebra: nothing here feeds a decision, so contraction is allowed.
-template <int AUXM>
+template <int AUXM, bool DET>
 __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<AUXM> &in, const BounceAcc<AUXM> &run,
                                              int g, uint32_t pidx, float Tp, float alpha, float G, float w, float dpt,
                                              F3 xyz, const F3 (&R)[3], float u, float v, float sx, float sy, F3 mean,
                                              float q0, float q1, float q2, float q3, float opac, float nsign,
                                              F3 normal, const float (&col)[3], const bool (&neg)[3], F3 ro, F3 rd,
                                              const float *__restrict__ sh, F3 &g_ro, F3 &g_rd,
-                                             const GradSink<AUXM> &sink, bool did, LastShHit &last) {
+                                             const GradSink<AUXM, DET> &sink, bool did, LastShHit &last) {
 #pragma clang fp contract(fast)
     // gradient algebra only: divisions become multiplications by a hardware reciprocal (1 ulp)
     const float num = 1.0f - alpha, inv_num = __builtin_amdgcn_rcpf(num);
@@ -1036,29 +1066,38 @@ __device__ __forceinline__ const uint64_t *rec_open(const RecView &rv, uint32_t 
 // Block-wide: write the table to the caller's gradient tensors and empty it.  Consecutive threads take
 // consecutive columns of a row, so the 48 SH columns of a surfel go out as contiguous atomics.  The caller
 // puts barriers around it.
-template <int AUXM>
+template <int AUXM, bool DET>
 __device__ __forceinline__ void table_flush(const DstParams &p, uint32_t *keys, float *rows) {
-    constexpr int stride = RowLayout<AUXM>::stride, n_rows = RowLayout<AUXM>::rows;
+    constexpr int stride = RowLayout<AUXM>::stride, n_rows = TableRows<AUXM, DET>::rows;
     for (int k = threadIdx.x; k < n_rows * stride; k += kWavesPerBlock * DST_WAVE) {
         const int row = k / stride, col = k - row * stride;
         const uint32_t g = keys[row];
         if (g == kEmptyKey || col >= RowLayout<AUXM>::cols) continue;
-        const float v = rows[k];
-        if (v == 0.f) continue;
-        rows[k] = 0.f;
-        float *dst = grad_address<AUXM>(p, g, col);
-        if (dst != nullptr) aadd(dst, v);
+        if (DET) {
+            long long *qrows = reinterpret_cast<long long *>(rows);
+            const long long q = qrows[k];
+            if (q == 0) continue;
+            qrows[k] = 0;
+            if (grad_address<AUXM>(p, g, col) != nullptr)
+                atomicAdd(p.det_workspace + (size_t)g * RowLayout<AUXM>::cols + col, (unsigned long long)q);
+        } else {
+            const float v = rows[k];
+            if (v == 0.f) continue;
+            rows[k] = 0.f;
+            float *dst = grad_address<AUXM>(p, g, col);
+            if (dst != nullptr) aadd(dst, v);
+        }
     }
 }
-template <int AUXM>
+template <int AUXM, bool DET>
 __device__ __forceinline__ void table_clear_keys(uint32_t *keys) {
-    for (int k = threadIdx.x; k <= RowLayout<AUXM>::rows; k += kWavesPerBlock * DST_WAVE)
-        keys[k] = (k < RowLayout<AUXM>::rows) ? kEmptyKey : 0u;
+    for (int k = threadIdx.x; k <= TableRows<AUXM, DET>::rows; k += kWavesPerBlock * DST_WAVE)
+        keys[k] = (k < TableRows<AUXM, DET>::rows) ? kEmptyKey : 0u;
 }
 
 // One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
 // and for BWD the per-hit gradients of the re-trace (reference backward.cu:332-655).
-template <bool BWD, int AUXM, bool REC, bool MIXED>
+template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
 __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
@@ -1233,10 +1272,11 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 Tp = Tn;
             } while (false);
             if (REC && BWD) fetch_geometry(want_next);
-            if (!BWD && p.training && p.a_weights != nullptr) wave_add_grouped(p.a_weights, did, (uint32_t)g, w);
+            if (!BWD && p.training && p.a_weights != nullptr)
+                wave_add_grouped(p.a_weights, (p.flags & DST_FLAG_DETERMINISTIC) ? p.det_workspace : nullptr, did, (uint32_t)g, w);
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
             if (BWD && wave_ballot(did) != 0ull) {
-                GradSink<AUXM> sink;
+                GradSink<AUXM, DET> sink;
                 sink.p = &p;
                 sink.rows = tab_rows;
                 sink.stage = stage;
@@ -1248,7 +1288,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 STAT(unsigned long long d1 = __builtin_readcyclecounter(); ws.t_plan += d1 - d0; ws.steps++;
                      ws.nodes += __popcll(wave_ballot(did && sink.own_slot < 0)); ws.leaves += __popcll(wave_ballot(sink.stray));
                      ws.leaf_any += __popcll(wave_ballot(did));)
-                hit_backward<AUXM>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
+                hit_backward<AUXM, DET>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
                                    q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did, last_sh);
                 STAT(ws.t_hb += __builtin_readcyclecounter() - d1;)
             }
@@ -1268,10 +1308,10 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         } while (false);
         if (BWD) {
             __syncthreads();   // every wave's additions of this round are in the table
-            if (tab_keys[RowLayout<AUXM>::rows] > (uint32_t)(3 * RowLayout<AUXM>::rows / 4)) {
-                table_flush<AUXM>(p, tab_keys, tab_rows);
+            if (tab_keys[TableRows<AUXM, DET>::rows] > (uint32_t)(3 * TableRows<AUXM, DET>::rows / 4)) {
+                table_flush<AUXM, DET>(p, tab_keys, tab_rows);
                 __syncthreads();
-                table_clear_keys<AUXM>(tab_keys);   // the barrier at the top of the next round publishes it
+                table_clear_keys<AUXM, DET>(tab_keys);   // the barrier at the top of the next round publishes it
             }
         }
     }
@@ -1304,14 +1344,14 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
     return v;
 }
 
-template <bool BWD, int AUXM, bool REC, bool MIXED>
+template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     constexpr int kTableRows = RowLayout<AUXM>::rows;
     __shared__ uint32_t s_keys[BWD ? kTableRows + 1 : 1];   // + the count of claimed rows
-    __shared__ float s_rows[BWD ? kTableRows * RowLayout<AUXM>::stride : 1];
+    __shared__ __attribute__((aligned(8))) float s_rows[BWD ? kTableRows * RowLayout<AUXM>::stride : 1];   // DET: half the rows, 8 bytes each
     __shared__ float s_stage[BWD ? kWavesPerBlock * kStageWords : 1];
     uint32_t *tab_keys = s_keys;
     float *tab_rows = s_rows;
@@ -1323,7 +1363,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         if (REC != complete) return;
     }
     if (BWD) {
-        table_clear_keys<AUXM>(s_keys);
+        table_clear_keys<AUXM, DET>(s_keys);
         for (int k = threadIdx.x; k < kTableRows * RowLayout<AUXM>::stride; k += kWavesPerBlock * DST_WAVE)
             s_rows[k] = 0.f;
         __syncthreads();
@@ -1384,7 +1424,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM, REC, MIXED>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i WS_ARG);
+            walk_bounce<false, AUXM, REC, MIXED, false>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -1527,7 +1567,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM, REC, MIXED>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
+            walk_bounce<true, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
         }
 #ifdef DST_STATS   // development build only: counters must then hold 11 entries
         if (p.counters != nullptr && lane == 0) {
@@ -1547,7 +1587,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             p.dL_dray_d[3 * r + 0] = g_rd.x; p.dL_dray_d[3 * r + 1] = g_rd.y; p.dL_dray_d[3 * r + 2] = g_rd.z;
         }
         __syncthreads();
-        table_flush<AUXM>(p, s_keys, s_rows);
+        table_flush<AUXM, DET>(p, s_keys, s_rows);
     }
 }
 
@@ -1563,13 +1603,34 @@ template <int AUXM, bool REC, bool MIXED>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x) {
-    trace_body<false, AUXM, REC, MIXED>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+    trace_body<false, AUXM, REC, MIXED, false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
 }
-template <int AUXM, bool REC, bool MIXED>
+template <int AUXM, bool REC, bool MIXED, bool DET>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
 void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x) {
-    trace_body<true, AUXM, REC, MIXED>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+}
+
+// Closing kernels of the deterministic mode: fixed point -> fp32, added to the caller's (zero-filled) tensors.
+template <int AUXM>
+__global__ void k_det_finish_grads(const DstParams p) {
+    constexpr int cols = RowLayout<AUXM>::cols;
+    const size_t n = (size_t)p.P * cols;
+    for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < n; k += (size_t)gridDim.x * blockDim.x) {
+        const long long q = (long long)p.det_workspace[k];
+        if (q == 0) continue;
+        const uint32_t g = (uint32_t)(k / cols);
+        const int col = (int)(k - (size_t)g * cols);
+        float *dst = grad_address<AUXM>(p, g, col);
+        if (dst != nullptr) *dst += from_fixed(q, det_shift(col));
+    }
+}
+__global__ void k_det_finish_weights(const DstParams p) {
+    for (int g = blockIdx.x * blockDim.x + threadIdx.x; g < p.P; g += gridDim.x * blockDim.x) {
+        const long long q = (long long)p.det_workspace[g];
+        if (q != 0) p.a_weights[g] += from_fixed(q, kDetShiftOther);
+    }
 }
 
 struct TileGrid {
@@ -1601,11 +1662,15 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipS
     // The per-lane walk is built into the kernels used where waves of unrelated rays are to be expected:
     // reflection bounces and ray lists (thin grids).  Image-shaped grids traced to depth 0 get the pure packet kernels.
     const bool mixed = p.max_trace_depth > 0 || t.th_log2 < 3;
+    const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
 #define DST_LAUNCH_M(AUX, MIXED)                                                                                   \
     do {                                                                                                           \
-        if (BWD)                                                                                                   \
-            hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC>), grid, block, 0, stream, p, acc, t.tw_log2, \
-                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                                       \
+        if (BWD && det)                                                                                            \
+            hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, true>), grid, block, 0, stream, p, acc,      \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                            \
+        else if (BWD)                                                                                              \
+            hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, false>), grid, block, 0, stream, p, acc,     \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                            \
         else                                                                                                       \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED>), grid, block, 0, stream, p, acc, t.tw_log2,          \
                                t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                                       \
@@ -1623,6 +1688,13 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipS
 }
 
 }  // namespace
+
+uint64_t dst_det_workspace_words(int32_t P, int32_t aux, int backward) {
+    if (P <= 0 || aux < 1 || aux > DST_MAX_AUX) return 0;
+    if (!backward) return (uint64_t)P;
+    const int cols = aux <= 2 ? RowLayout<2>::cols : (aux <= 4 ? RowLayout<4>::cols : RowLayout<8>::cols);
+    return (uint64_t)P * cols;
+}
 
 uint64_t dst_hit_record_layout(int32_t H, int32_t W, int32_t mtd_alloc, uint32_t blocks, uint64_t *header_words,
                                uint32_t *n_waves) {
@@ -1651,12 +1723,21 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     acc.n_leaves = ctx->n_leaves;
     acc.root = dst_root_ref(ctx->n_leaves);
     const bool rec = p.hit_record != nullptr;
+    const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
     if (backward) {
         if (rec) launch<true, true>(p, acc, t, stream);   // does the work if the record is complete,
         launch<true, false>(p, acc, t, stream);           // else this one does (it returns at once otherwise)
+        if (det) {
+            const dim3 grid(2048), block(256);
+            if (p.aux <= 2) hipLaunchKernelGGL(k_det_finish_grads<2>, grid, block, 0, stream, p);
+            else if (p.aux <= 4) hipLaunchKernelGGL(k_det_finish_grads<4>, grid, block, 0, stream, p);
+            else hipLaunchKernelGGL(k_det_finish_grads<8>, grid, block, 0, stream, p);
+        }
     } else {
         if (rec) launch<false, true>(p, acc, t, stream);
         else launch<false, false>(p, acc, t, stream);
+        if (det && p.training && p.a_weights != nullptr)
+            hipLaunchKernelGGL(k_det_finish_weights, dim3(1024), dim3(256), 0, stream, p);
     }
     DST_HIP(ctx, hipGetLastError());
     return DST_OK;

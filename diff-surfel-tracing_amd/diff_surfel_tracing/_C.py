@@ -16,6 +16,7 @@ DEFAULT_AUX_CHANNELS = 2  # reference optix_tracer/config.h:6
 DEFAULT_MAX_TRACE_DEPTH = 1  # reference optix_tracer/config.h:27: mid_val always holds at least two slots
 MAX_AUX_CHANNELS = 8
 MAX_TRACE_DEPTH = 3
+FLAG_DETERMINISTIC = 1
 
 _FP = C.c_void_p
 
@@ -30,7 +31,7 @@ class DstParams(C.Structure):
                               "others_precomp", "opacities", "scales", "rotations")]
         + [(n, _FP) for n in ("out_rgb", "out_dpt", "out_acc", "out_norm", "out_dist", "out_aux", "mid_val",
                               "a_weights", "counters", "hit_record")]
-        + [("hit_record_blocks", C.c_uint32), ("reserved0", C.c_uint32)]
+        + [("hit_record_blocks", C.c_uint32), ("flags", C.c_uint32), ("det_workspace", _FP)]
         + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
         + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
                               "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
@@ -45,7 +46,8 @@ class DstAccelInfo(C.Structure):
 
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
            "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params",
-           "dst_hit_record_layout", "dst_refit_accel_static", "dst_refit_from_surfels")
+           "dst_hit_record_layout", "dst_refit_accel_static", "dst_refit_from_surfels",
+           "dst_det_workspace_words")
 
 _lib = None
 
@@ -73,6 +75,8 @@ def load_library():
     L.dst_last_error.argtypes = [C.c_void_p]
     L.dst_accel_info.argtypes = [C.c_void_p, C.POINTER(DstAccelInfo)]
     L.dst_accel_download.argtypes = [C.c_void_p] * 7
+    L.dst_det_workspace_words.restype = C.c_uint64
+    L.dst_det_workspace_words.argtypes = [C.c_int32, C.c_int32, C.c_int]
     L.dst_version.restype = C.c_char_p
     L.dst_sizeof_params.restype = C.c_size_t
     L.dst_hit_record_layout.restype = C.c_uint64
@@ -189,6 +193,7 @@ class OptiXStateWrapper:
         self.record_blocks_per_wave = 6.0   # sizing estimate for hit records, raised when a record overflows
         self.record_max_bytes = 8 << 30     # no record larger than this is made (backward then re-traces)
         self.record_wanted = True           # set by the autograd wrapper for the call that follows
+        self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
         self._record_pool = []              # free storages (int64 tensors)
         self._record_fixed = False          # True: only caller-provided storage is used, nothing is allocated
         self._record_watch = []             # records whose request count has not been read yet
@@ -349,6 +354,10 @@ def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, backg
     p.counters = _ptr(counters)
     if hit_record is not None:
         p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
+    det_ws = None
+    if getattr(ctx, "deterministic", False) and training:
+        det_ws = torch.zeros(load_library().dst_det_workspace_words(P, p.aux, 0), dtype=torch.int64, device=dev)
+        p.flags, p.det_workspace = FLAG_DETERMINISTIC, det_ws.data_ptr()
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))
@@ -407,6 +416,10 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
         # nothing here waits for the forward trace
         p.hit_record, p.hit_record_blocks = hit_record.words.data_ptr(), hit_record.blocks
     p.counters = _ptr(counters)
+    det_ws = None
+    if getattr(ctx, "deterministic", False):
+        det_ws = torch.zeros(load_library().dst_det_workspace_words(P, p.aux, 1), dtype=torch.int64, device=dev)
+        p.flags, p.det_workspace = FLAG_DETERMINISTIC, det_ws.data_ptr()
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))

@@ -137,6 +137,17 @@ class SurfelTracer(nn.Module):
         # keeps the reference's attribute name; owns the BVH instead of an OptiX pipeline
         self.optix_context = _C.OptiXStateWrapper(self.pkg_dir)
 
+    @property
+    def deterministic(self) -> bool:
+        """Extension (not in the reference): when set, the accumulated blending weights and all per-surfel
+        gradients are summed in 64-bit fixed point (exact, order-independent) instead of with float atomics: the
+        same inputs give the same bits on every run.  Costs time and a workspace of 8 bytes per sum."""
+        return self.optix_context.deterministic
+
+    @deterministic.setter
+    def deterministic(self, value: bool) -> None:
+        self.optix_context.deterministic = bool(value)
+
     def build_acceleration_structure(self, vertices: torch.Tensor, triangles: torch.Tensor, rebuild: bool = 1):
         """Build (`rebuild` true) or refit in place the BVH over the surfel quads `vertices` (4P,3), `triangles` (2P,3)."""
         return _C.build_acceleration_structure(self.optix_context, vertices, triangles, rebuild)

@@ -35,6 +35,8 @@ enum {
     DST_E_UNSUPPORTED = 5  /* setting outside what the kernels are instantiated for */
 };
 
+#define DST_FLAG_DETERMINISTIC 1u /* bitwise reproducible a_weights (forward) and per-surfel gradients (backward) */
+
 #define DST_MAX_AUX 8        /* auxiliary channels per surfel (reference AUX_CHANNELS = 2) */
 #define DST_MAX_TRACE_DEPTH 3 /* bounces after the primary ray (reference MAX_TRACE_DEPTH = 1) */
 #define DST_STATIC_REFIT_MAX_SURFELS (1u << 21) /* largest structure dst_refit_accel_static serves */
@@ -89,7 +91,13 @@ typedef struct DstParams {
      * not written by a forward trace with the same grid, depth and a zeroed header. */
     uint64_t *hit_record;
     uint32_t hit_record_blocks;
-    uint32_t reserved0;
+    uint32_t flags;               /* DST_FLAG_* */
+    /* workspace of the deterministic mode (DST_FLAG_DETERMINISTIC; no counterpart in the reference, whose float
+     * atomics make a_weights and the per-surfel gradients depend on the order in which rays finish): every
+     * atomically accumulated sum is formed in 64-bit fixed point, where addition is exact and hence independent of
+     * order, in this buffer, and converted to fp32 into the caller's tensor by a closing kernel of the same call.
+     * Device memory, dst_det_workspace_words() 8-byte words, zero-filled by the caller before each call. */
+    unsigned long long *det_workspace;
     /* upstream gradients (backward) */
     const float *dL_drgb, *dL_ddpt, *dL_dacc, *dL_ddist, *dL_dnorm, *dL_daux;
     /* gradient outputs; the per-surfel ones are ACCUMULATED into: caller zero-fills */
@@ -178,6 +186,10 @@ int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_p
  * grid is traced with (a forward trace at depth 0 asks for about 3-6 blocks per wave). */
 uint64_t dst_hit_record_layout(int32_t H, int32_t W, int32_t mtd_alloc, uint32_t blocks, uint64_t *header_words,
                                uint32_t *n_waves);
+
+/* Words (8 bytes each) of DstParams.det_workspace for a forward (backward = 0: one per surfel) or a backward
+ * call (one per surfel and gradient column: 16 + aux table columns + 48 SH columns). */
+uint64_t dst_det_workspace_words(int32_t P, int32_t aux, int backward);
 
 /* Library version string, and sizeof(DstParams) as compiled (lets a foreign-language binding
  * verify its own struct layout before the first launch). */
