@@ -34,7 +34,8 @@ int check_common(dst_ctx *ctx, const DstParams *p) {
                         "vertices, background, means3D, opacities, scales and rotations are required");
     if ((p->flags & DST_FLAG_DETERMINISTIC) && !p->det_workspace)
         return dst_fail(ctx, DST_E_INVALID, "the deterministic mode needs det_workspace");
-    if (p->flags & ~DST_FLAG_DETERMINISTIC) return dst_fail(ctx, DST_E_INVALID, "unknown bits in flags");
+    if (p->flags & ~(DST_FLAG_DETERMINISTIC | DST_FLAG_DISTORTION))
+        return dst_fail(ctx, DST_E_INVALID, "unknown bits in flags");
     if (p->hit_record && (reinterpret_cast<uintptr_t>(p->hit_record) & 7u))
         return dst_fail(ctx, DST_E_INVALID, "hit_record must be 8-byte aligned");
     if (p->H > 0 && p->W > 0 &&

@@ -20,6 +20,7 @@ constexpr double kStepEps = 0.00001;
 constexpr int kMaxContrib = 256;
 constexpr float kStartOffset = 0.06f;
 constexpr float kNear = 0.2f;
+constexpr float kFar = 100.0f;   // reference auxiliary.h:20-21
 constexpr float kTmin = 0.0001f;
 constexpr int kWavesPerBlock = 4;
 #ifndef DST_FWD_WPB
@@ -1102,7 +1103,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
                                             uint32_t &n_con, uint32_t *tab_keys, float *tab_rows, float *stage,
-                                            const RecView &rv, int bounce
+                                            const RecView &rv, int bounce, F3 &dist_acc
 #ifdef DST_STATS
                                             , WaveStats &ws
 #endif
@@ -1259,6 +1260,15 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
 #pragma unroll
                     for (int ch = 0; ch < AUXM; ++ch)
                         if (ch < p.aux) run.O[ch] += w * p.others_precomp[(size_t)p.aux * g + ch];
+                }
+                if (!BWD && (p.flags & DST_FLAG_DISTORTION)) {
+                    // depth distortion of 2DGS with its running moments (x = distortion, y = M1, z = M2); the
+                    // reference declares the three and leaves the computation open (forward.cu:286)
+                    const float A_before = 1 - Tp;
+                    const float m = kFar / (kFar - kNear) * (1 - kNear / dpt);
+                    dist_acc.x += (m * m * A_before + dist_acc.z - 2 * m * dist_acc.y) * w;
+                    dist_acc.y += m * w;
+                    dist_acc.z += m * m * w;
                 }
                 run.D += w * dpt;
                 run.N[0] += w * normal.x;
@@ -1424,7 +1434,8 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         bool on = inside;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<false, AUXM, REC, MIXED, false>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i WS_ARG);
+            F3 dist_acc = f3(0, 0, 0);
+            walk_bounce<false, AUXM, REC, MIXED, false>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i, dist_acc WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -1437,9 +1448,9 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                     p.out_norm[3 * r + 0] = run.N[0];
                     p.out_norm[3 * r + 1] = run.N[1];
                     p.out_norm[3 * r + 2] = run.N[2];
-                    p.out_dist[3 * r + 0] = 0.f;
-                    p.out_dist[3 * r + 1] = 0.f;
-                    p.out_dist[3 * r + 2] = 0.f;
+                    p.out_dist[3 * r + 0] = dist_acc.x;   // zeros unless DST_FLAG_DISTORTION (as the reference)
+                    p.out_dist[3 * r + 1] = dist_acc.y;
+                    p.out_dist[3 * r + 2] = dist_acc.z;
 #pragma unroll
                     for (int ch = 0; ch < AUXM; ++ch)
                         if (ch < p.aux) p.out_aux[(size_t)p.aux * r + ch] = run.O[ch];
@@ -1567,7 +1578,8 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
                 }
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
-            walk_bounce<true, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i WS_ARG);
+            F3 no_dist = f3(0, 0, 0);
+            walk_bounce<true, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i, no_dist WS_ARG);
         }
 #ifdef DST_STATS   // development build only: counters must then hold 11 entries
         if (p.counters != nullptr && lane == 0) {

@@ -17,6 +17,7 @@ DEFAULT_MAX_TRACE_DEPTH = 1  # reference optix_tracer/config.h:27: mid_val alway
 MAX_AUX_CHANNELS = 8
 MAX_TRACE_DEPTH = 3
 FLAG_DETERMINISTIC = 1
+FLAG_DISTORTION = 2
 
 _FP = C.c_void_p
 
@@ -194,6 +195,7 @@ class OptiXStateWrapper:
         self.record_max_bytes = 8 << 30     # no record larger than this is made (backward then re-traces)
         self.record_wanted = True           # set by the autograd wrapper for the call that follows
         self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
+        self.distortion = False             # True: the dist output carries the 2DGS depth distortion (else zeros)
         self._record_pool = []              # free storages (int64 tensors)
         self._record_fixed = False          # True: only caller-provided storage is used, nothing is allocated
         self._record_watch = []             # records whose request count has not been read yet
@@ -358,6 +360,8 @@ def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, backg
     if getattr(ctx, "deterministic", False) and training:
         det_ws = torch.zeros(load_library().dst_det_workspace_words(P, p.aux, 0), dtype=torch.int64, device=dev)
         p.flags, p.det_workspace = FLAG_DETERMINISTIC, det_ws.data_ptr()
+    if getattr(ctx, "distortion", False):
+        p.flags |= FLAG_DISTORTION
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))

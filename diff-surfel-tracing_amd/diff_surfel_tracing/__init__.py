@@ -148,6 +148,17 @@ class SurfelTracer(nn.Module):
     def deterministic(self, value: bool) -> None:
         self.optix_context.deterministic = bool(value)
 
+    @property
+    def distortion(self) -> bool:
+        """Extension (not in the reference, which returns zeros: forward.cu:286): when set, the `dist` output is the
+        depth distortion of the primary ray as 2DGS defines it, sum_i sum_{j<i} w_i w_j (m_i - m_j)^2 with
+        m = far/(far-near) (1 - near/depth), near 0.2, far 100.  Forward only: no gradient flows from it."""
+        return self.optix_context.distortion
+
+    @distortion.setter
+    def distortion(self, value: bool) -> None:
+        self.optix_context.distortion = bool(value)
+
     def build_acceleration_structure(self, vertices: torch.Tensor, triangles: torch.Tensor, rebuild: bool = 1):
         """Build (`rebuild` true) or refit in place the BVH over the surfel quads `vertices` (4P,3), `triangles` (2P,3)."""
         return _C.build_acceleration_structure(self.optix_context, vertices, triangles, rebuild)

@@ -36,6 +36,10 @@ enum {
 };
 
 #define DST_FLAG_DETERMINISTIC 1u /* bitwise reproducible a_weights (forward) and per-surfel gradients (backward) */
+#define DST_FLAG_DISTORTION 2u    /* forward: out_dist = (depth distortion, M1, M2) of the primary ray as 2DGS defines
+                                   * them; the reference leaves it at zero (forward.cu:286) and so does this library
+                                   * without the flag.  No gradient flows from it (the reference's backward never reads
+                                   * dL_ddist either). */
 
 #define DST_MAX_AUX 8        /* auxiliary channels per surfel (reference AUX_CHANNELS = 2) */
 #define DST_MAX_TRACE_DEPTH 3 /* bounces after the primary ray (reference MAX_TRACE_DEPTH = 1) */

@@ -75,6 +75,7 @@ constexpr double kStepEps = 0.00001;
 constexpr int kMaxContrib = 256;
 constexpr float kStartOffset = 0.06f;
 constexpr float kNear = 0.2f;
+constexpr float kFar = 100.0f;  // auxiliary.h:20-21
 constexpr float kTmin = 0.0001f;
 constexpr int kMaxAux = 8;
 constexpr int kMaxSlots = 4;  // mtd_alloc + 1
@@ -484,6 +485,7 @@ void flush(const std::vector<double> &a, float *out) {
 struct BounceOut {
     float C[3], D, A, O[kMaxAux], T;
     V3 N, E;
+    float DS, M1, M2;   // depth distortion and its running moments (only with compute_dist)
 };
 
 inline int mid_channels(const OracleParams *p) { return 11 + p->aux + 3; }
@@ -503,6 +505,7 @@ void bounce_forward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float 
     for (int ch = 0; ch < kMaxAux; ++ch) r.O[ch] = 0.f;
     r.D = 0.f;
     r.N = v3(0, 0, 0);
+    r.DS = r.M1 = r.M2 = 0.f;
     for (;;) {
         k_nearest(sc, ray_ot, ray_d, buf, pay_cnt);
         int contributed_here = 0;
@@ -548,6 +551,14 @@ void bounce_forward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float 
             }
             if (p->others_precomp != nullptr)
                 for (int ch = 0; ch < p->aux; ++ch) r.O[ch] += w * p->others_precomp[ch + (size_t)p->aux * g];
+            if (p->compute_dist) {
+                // the distortion the reference declares and leaves open (forward.cu:147-152,286), as 2DGS defines it
+                const float A_before = 1 - T_prev;
+                const float m = kFar / (kFar - kNear) * (1 - kNear / dpt);
+                r.DS += (m * m * A_before + r.M2 - 2 * m * r.M1) * w;
+                r.M1 += m * w;
+                r.M2 += m * m * w;
+            }
             r.D += w * dpt;
             r.N = v3(r.N.x + w * normal.x, r.N.y + w * normal.y, r.N.z + w * normal.z);
             T_prev = T_next;
@@ -570,7 +581,7 @@ void bounce_forward(const Scene &sc, V3 ray_o, V3 ray_d, float min_depth, float 
 
 // forward.cu:318-424
 void path_forward(const Scene &sc, V3 ray_o, V3 ray_d, float *out_rgb, float &out_dpt, float &out_acc, V3 &out_norm,
-                  float *out_aux, float *mid, Accum *acc, int &n_proc, int &n_con) {
+                  V3 &out_dist, float *out_aux, float *mid, Accum *acc, int &n_proc, int &n_con) {
     const OracleParams *p = sc.p;
     const int MID = mid_channels(p), AUXO = 11, RGBO = 11 + p->aux;
     V3 ot = ray_o, dt = ray_d;
@@ -583,6 +594,7 @@ void path_forward(const Scene &sc, V3 ray_o, V3 ray_d, float *out_rgb, float &ou
             out_dpt = b.D;
             out_acc = b.A;
             out_norm = b.N;
+            out_dist = v3(b.DS, b.M1, b.M2);   // forward.cu:384 (zeros in the reference: never accumulated)
             for (int ch = 0; ch < p->aux; ++ch) out_aux[ch] = b.O[ch];
         }
         float f_this = (i == p->max_trace_depth) ? 1.0f : 1 - b.O[0];
@@ -997,16 +1009,16 @@ int oracle_trace_forward(const OracleParams *p) {
     for (long r = 0; r < R; ++r) {
         V3 o = ld3(p->ray_o + 3 * r), d = ld3(p->ray_d + 3 * r);
         float rgb[3] = {0, 0, 0}, dptv = 0.f, accv = 0.f, aux[kMaxAux] = {0};
-        V3 nrm = v3(0, 0, 0);
+        V3 nrm = v3(0, 0, 0), dist = v3(0, 0, 0);
         float mid[kMaxSlots * (14 + kMaxAux)];
         for (float &m : mid) m = 0.f;
         int n_proc = 0, n_con = 0;
-        path_forward(sc, o, d, rgb, dptv, accv, nrm, aux, mid, accp, n_proc, n_con);
+        path_forward(sc, o, d, rgb, dptv, accv, nrm, dist, aux, mid, accp, n_proc, n_con);
         for (int ch = 0; ch < 3; ++ch) p->out_rgb[3 * r + ch] = rgb[ch];
         p->out_dpt[r] = dptv;
         p->out_acc[r] = accv;
         p->out_norm[3 * r + 0] = nrm.x; p->out_norm[3 * r + 1] = nrm.y; p->out_norm[3 * r + 2] = nrm.z;
-        for (int ch = 0; ch < 3; ++ch) p->out_dist[3 * r + ch] = 0.f;
+        p->out_dist[3 * r + 0] = dist.x; p->out_dist[3 * r + 1] = dist.y; p->out_dist[3 * r + 2] = dist.z;
         for (int ch = 0; ch < p->aux; ++ch) p->out_aux[(size_t)p->aux * r + ch] = aux[ch];
         for (int i = 0; i < slots * MID; ++i)
             p->mid_val[(size_t)slots * MID * r + i] = (i < (p->max_trace_depth + 1) * MID) ? mid[i] : 0.f;

@@ -52,6 +52,10 @@ typedef struct OracleParams {
     int32_t hit_mode;      /* ORACLE_HITS_* */
     int32_t literal_stale; /* 1: keep the reference's stale slot on a repeated surfel (forward.cu:207-208) */
     int32_t n_threads;     /* OpenMP threads, 0 = default */
+    int32_t compute_dist;  /* forward only.  0: out_dist stays zero, as in the reference (forward.cu:286 leaves the
+                            * accumulation open).  1: out_dist = (depth distortion, M1, M2) of the primary ray as 2DGS
+                            * defines them: dist += (m*m*(1-T) + M2 - 2*m*M1)*w, M1 += m*w, M2 += m*m*w with
+                            * m = far/(far-near)*(1-near/depth), near 0.2, far 100 (auxiliary.h:20-21) */
     int32_t grad_f64;      /* backward only.  0: gradient algebra in float, operation by operation as the reference
                             * writes it (the restatement).  1: the same formulas in double on the same fp32 inputs,
                             * hits and decisions; the difference between the two shows how much of a float gradient

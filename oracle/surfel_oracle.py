@@ -24,7 +24,7 @@ class OracleParams(C.Structure):
         [(n, C.c_int32) for n in ("P", "H", "W", "D", "M", "aux", "mtd_alloc", "training", "start_from_first",
                                   "max_trace_depth")]
         + [("specular_threshold", C.c_float)]
-        + [(n, C.c_int32) for n in ("hit_mode", "literal_stale", "n_threads", "grad_f64")]
+        + [(n, C.c_int32) for n in ("hit_mode", "literal_stale", "n_threads", "compute_dist", "grad_f64")]
         + [("ray_o", _FP), ("ray_d", _FP), ("vertices", _FP), ("faces", _IP)]
         + [(n, _FP) for n in ("background", "means3D", "shs", "colors_precomp", "others_precomp", "opacities",
                               "scales", "rotations")]
@@ -120,8 +120,9 @@ class Scene:
         return p
 
 
-def forward(sc, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0, counters=True):
-    """Run the oracle forward.  Returns a dict of numpy arrays shaped like the reference outputs."""
+def forward(sc, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0, counters=True, compute_dist=False):
+    """Run the oracle forward.  Returns a dict of numpy arrays shaped like the reference outputs.  `compute_dist`:
+    fill "dist" with the 2DGS depth distortion and its two moments instead of the reference's zeros."""
     H, W, P = sc.H, sc.W, sc.P
     MID = 14 + sc.aux
     out = {
@@ -135,6 +136,7 @@ def forward(sc, hit_mode=HITS_BRUTE_LEXI, literal_stale=False, n_threads=0, coun
         out["n_proc"] = np.zeros((H, W), np.int32)
         out["n_con"] = np.zeros((H, W), np.int32)
     p = sc.params(hit_mode, literal_stale, n_threads)
+    p.compute_dist = int(bool(compute_dist))
     p.out_rgb, p.out_dpt, p.out_acc = _fp(out["rgb"]), _fp(out["dpt"]), _fp(out["acc"])
     p.out_norm, p.out_dist, p.out_aux = _fp(out["norm"]), _fp(out["dist"]), _fp(out["aux"])
     p.mid_val = _fp(out["mid"])

@@ -262,3 +262,22 @@ def test_raw_launcher_calls_without_a_record(oracle, tracer):
     got = {k: t.cpu().numpy() for t, k in zip(bwd, names) if k is not None}
     assert_gradients(got, {k: refg[k] for k in got}, refg64, GRAD_REL)
     assert bwd[4].abs().max() == 0 and bwd[11].shape == (3000, 9) and bwd[11].abs().max() == 0
+
+
+def test_distortion_output_is_opt_in_and_equals_the_oracle(oracle, tracer):
+    """`dist` is zero as in the reference unless SurfelTracer.distortion is set; then it is the 2DGS depth distortion
+    of the primary ray, bit-equal to the oracle's, and nothing else changes."""
+    sc = S.scene_cube(P=6000, seed=12)
+    o, d = S.rays_cube(56, 72)
+    s = oracle_scene(oracle, sc, o, d)
+    ref = oracle.forward(s, oracle.HITS_BVH_LEXI, compute_dist=True)
+    plain, _ = gpu_trace(tracer, sc, o, d)
+    assert (plain["dist"] == 0).all()
+    tracer.distortion = True
+    try:
+        out, g = gpu_trace(tracer, sc, o, d, upstream=upstream(56, 72, 2))
+    finally:
+        tracer.distortion = False
+    assert_forward_exact({**out, "dist": plain["dist"]}, {**ref, "dist": np.zeros_like(ref["dist"])})
+    np.testing.assert_array_equal(out["dist"].view(np.uint32), ref["dist"][..., :1].view(np.uint32))
+    assert out["dist"].max() > 1e-6 and g["means3D"] is not None

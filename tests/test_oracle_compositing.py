@@ -278,3 +278,36 @@ def test_malformed_requests_are_rejected(oracle):
     bad["faces"][1, 0] = 3
     with pytest.raises(RuntimeError):
         oracle.forward(oracle_scene(oracle, bad, o, d))
+
+
+def test_depth_distortion_is_the_pairwise_sum_it_stands_for(oracle):
+    """compute_dist (an extension: the reference leaves `dist` at zero, forward.cu:286): the running-moment form
+    equals sum_i sum_{j<i} w_i w_j (m_i - m_j)^2 with m = far/(far-near) (1 - near/depth); M1, M2 are the weighted
+    moments.  Checked against a float64 evaluation from the per-hit weights of the independent forward model."""
+    from test_oracle_gradients import forward64, make_case
+    sc, ro, rd, _ = make_case(7, P=80, R=50)
+    rd = rd / rd.norm(dim=-1, keepdim=True)       # unit directions: depth = distance
+    R = ro.shape[0]
+    s = oracle_scene(oracle, sc, ro.reshape(1, R, 3), rd.reshape(1, R, 3))
+    plain = oracle.forward(s, oracle.HITS_BRUTE_LEXI)
+    assert (plain["dist"] == 0).all()
+    out = oracle.forward(s, oracle.HITS_BRUTE_LEXI, compute_dist=True)
+    for k in ("rgb", "dpt", "acc", "norm", "aux", "mid"):
+        np.testing.assert_array_equal(out[k], plain[k])
+    leaf = {k: sc[k].double() for k in sc if k not in ("vertices", "faces")}
+    # per-hit depths in compositing order: recompute them from the model's weights (w) and ordered t
+    Rm = S.build_rotation(leaf["rotations"])
+    rgb, dpt, nrm, aux, info = forward64(ro.double(), rd.double(), leaf["means3D"], leaf["scales"], leaf["rotations"],
+                                         leaf["opacities"], torch.zeros(3, dtype=torch.float64),
+                                         colors=leaf["colors_precomp"], others=leaf["others_precomp"])
+    np.testing.assert_array_equal(out["n_con"].reshape(R), info["n_con"].numpy())
+    w, t = info["w"], info["t_sorted"]
+    m = 100.0 / (100.0 - 0.2) * (1 - 0.2 / t)
+    m = torch.where(w > 0, m, torch.zeros_like(m))
+    pair = (w[:, :, None] * w[:, None, :] * (m[:, :, None] - m[:, None, :]) ** 2)
+    want = torch.tril(pair, diagonal=-1).sum((1, 2))
+    got = out["dist"].reshape(R, 3)
+    np.testing.assert_allclose(got[:, 0], want.numpy(), rtol=2e-3, atol=1e-7)
+    np.testing.assert_allclose(got[:, 1], (w * m).sum(1).numpy(), rtol=1e-4, atol=1e-7)
+    np.testing.assert_allclose(got[:, 2], (w * m * m).sum(1).numpy(), rtol=1e-4, atol=1e-7)
+    assert want.max() > 1e-6

@@ -107,7 +107,7 @@ def forward64(ro, rd, means, scales, quats, opac, bg, colors=None, shs=None, oth
         oth = others[None].expand(ro.shape[0], -1, -1)
         aux = (w[..., None] * torch.gather(oth, 1, order[..., None].expand(-1, -1, others.shape[1]))).sum(1)
     edge = torch.where(in0 | in1, torch.where(in0, m0, m1), torch.minimum(m0, m1))
-    info = {"n_con": (w > 0).sum(1), "w": w, "alpha": a_s, "acc": w.sum(1), "edge_margin": torch.where(t > 0, edge, torch.ones_like(edge)).min(),
+    info = {"n_con": (w > 0).sum(1), "w": w, "alpha": a_s, "acc": w.sum(1), "t_sorted": gat(t), "edge_margin": torch.where(t > 0, edge, torch.ones_like(edge)).min(),
             "thresh_margin": torch.where(hit, (alpha - 1 / 255).abs(), torch.ones_like(alpha)).min()}
     return rgb, dpt, nrm, aux, info
 
