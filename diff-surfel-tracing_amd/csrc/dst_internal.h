@@ -101,6 +101,9 @@ struct dst_ctx {
     uint32_t *keys[2] = {nullptr, nullptr}, *vals[2] = {nullptr, nullptr};
     uint32_t *tile_hist = nullptr;
     size_t tile_hist_elems = 0;
+    // ordering of ray lists (thin ray grids): sort keys / ray numbers ping-pong and radix histograms, grow-only
+    uint32_t *ray_keys[2] = {nullptr, nullptr}, *ray_vals[2] = {nullptr, nullptr}, *ray_hist = nullptr;
+    uint32_t ray_capacity = 0;
     DstBounds *bounds = nullptr;       // device
     DstBounds *bounds_host = nullptr;  // pinned host copy
     float scene_lo[3] = {0, 0, 0}, scene_hi[3] = {0, 0, 0}, max_abs = 0;
@@ -126,6 +129,8 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
 int dst_static_scratch_init(dst_ctx *ctx);
 uint32_t *dst_static_scratch(const dst_ctx *ctx);
 void dst_lbvh_free(dst_ctx *ctx);
+void dst_sort_pairs(uint32_t *keys[2], uint32_t *vals[2], uint32_t *tile_hist, uint32_t n, hipStream_t stream);
+size_t dst_sort_hist_elems(uint32_t n);
 // trace.hip
 int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream);
 

@@ -610,6 +610,22 @@ uint32_t *dst_static_scratch(const dst_ctx *ctx) {
     return (ctx->device >= 0 && ctx->device < kMaxDevices) ? g_refit_scratch_ptr[ctx->device] : nullptr;
 }
 
+// Stable LSD radix sort of (key, value) pairs, 32-bit keys, four 8-bit passes; the sorted pairs end in buffer 0.
+// tile_hist holds 256 counters per 1024 keys.  Used by the BVH build (Morton codes) and by the ray ordering.
+void dst_sort_pairs(uint32_t *keys[2], uint32_t *vals[2], uint32_t *tile_hist, uint32_t n, hipStream_t stream) {
+    const uint32_t tiles = (n + kTile - 1) / kTile;
+    const uint32_t tile_blocks = (tiles + (kBlock / DST_WAVE) - 1) / (kBlock / DST_WAVE);
+    int src = 0;
+    for (int shift = 0; shift < 32; shift += kRadixBits) {
+        hipLaunchKernelGGL(k_radix_hist, dim3(tile_blocks), dim3(kBlock), 0, stream, keys[src], tile_hist, n, tiles, shift);
+        hipLaunchKernelGGL(k_scan_exclusive, dim3(1), dim3(1024), 0, stream, tile_hist, tiles * kRadix);
+        hipLaunchKernelGGL(k_radix_scatter, dim3(tile_blocks), dim3(kBlock), 0, stream, keys[src], vals[src],
+                           keys[1 - src], vals[1 - src], tile_hist, n, tiles, shift);
+        src = 1 - src;
+    }
+}
+size_t dst_sort_hist_elems(uint32_t n) { return (size_t)((n + kTile - 1) / kTile) * kRadix; }
+
 void dst_lbvh_free(dst_ctx *ctx) {
     auto rel = [](auto *&p) {
         if (p) (void)hipFree(p);
@@ -629,6 +645,12 @@ void dst_lbvh_free(dst_ctx *ctx) {
     rel(ctx->vals[0]);
     rel(ctx->vals[1]);
     rel(ctx->tile_hist);
+    rel(ctx->ray_keys[0]);
+    rel(ctx->ray_keys[1]);
+    rel(ctx->ray_vals[0]);
+    rel(ctx->ray_vals[1]);
+    rel(ctx->ray_hist);
+    ctx->ray_capacity = 0;
     ctx->capacity = 0;
     ctx->built = false;
     ctx->n_leaves = 0;
@@ -666,18 +688,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     if (rebuild) {
         hipLaunchKernelGGL(k_morton, grid_for(n), dim3(kBlock), 0, stream, centroids, ctx->bounds, ctx->keys[0],
                            ctx->vals[0], n);
-        const uint32_t tiles = (n + kTile - 1) / kTile;
-        const uint32_t tile_blocks = (tiles + (kBlock / DST_WAVE) - 1) / (kBlock / DST_WAVE);
-        int src = 0;
-        for (int shift = 0; shift < 32; shift += kRadixBits) {
-            hipLaunchKernelGGL(k_radix_hist, dim3(tile_blocks), dim3(kBlock), 0, stream, ctx->keys[src], ctx->tile_hist,
-                               n, tiles, shift);
-            hipLaunchKernelGGL(k_scan_exclusive, dim3(1), dim3(1024), 0, stream, ctx->tile_hist, tiles * kRadix);
-            hipLaunchKernelGGL(k_radix_scatter, dim3(tile_blocks), dim3(kBlock), 0, stream, ctx->keys[src],
-                               ctx->vals[src], ctx->keys[1 - src], ctx->vals[1 - src], ctx->tile_hist, n, tiles, shift);
-            src = 1 - src;
-        }
-        // four passes: the sorted pairs are back in buffer 0
+        dst_sort_pairs(ctx->keys, ctx->vals, ctx->tile_hist, n, stream);   // the sorted pairs end in buffer 0
         if (n > 1) {
             hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->node_parent, DST_NO_PARENT, n);
             hipLaunchKernelGGL(k_karras, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->keys[0], ctx->nodes,

@@ -432,7 +432,7 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
 // quad tests, same buffer.  The buffer's content does not depend on the order of arrival, so both walks give
 // the same result bit for bit; the choice between them only changes the time.
 #ifndef DST_PACKET_DIR_SPREAD
-#define DST_PACKET_DIR_SPREAD 0.06f
+#define DST_PACKET_DIR_SPREAD 0.02f   // measured: 0.06 makes packets of lidar rays that are metres apart at their hits
 #endif
 #ifndef DST_PACKET_ORG_SPREAD
 #define DST_PACKET_ORG_SPREAD 0.02f
@@ -1356,7 +1356,8 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
 
 template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
-                                           uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x) {
+                                           uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x,
+                                           const uint32_t *__restrict__ ray_order) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     constexpr int kTableRows = RowLayout<AUXM>::rows;
@@ -1409,7 +1410,9 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     const uint32_t py = (ty << th_log2) + (lane >> tw_log2);
     const uint32_t px = (tx << tw_log2) + (lane & ((1u << tw_log2) - 1u));
     const bool inside = wave_on && py < (uint32_t)p.H && px < (uint32_t)p.W;
-    const size_t r = inside ? ((size_t)py * p.W + px) : 0;
+    // ray lists are traced in a coherent order (see k_ray_keys): position in that order -> ray number
+    const size_t pos = inside ? ((size_t)py * p.W + px) : 0;
+    const size_t r = (ray_order != nullptr && inside) ? (size_t)ray_order[pos] : pos;
     const float max_abs = __uint_as_float(acc.bounds->max_abs);
     const int MID = 14 + p.aux, AUXO = 11, RGBO = 11 + p.aux;
     const int slots = p.mtd_alloc + 1, mtd = p.max_trace_depth;
@@ -1614,14 +1617,14 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
 template <int AUXM, bool REC, bool MIXED>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
-                 uint32_t tiles_y, uint32_t btiles_x) {
-    trace_body<false, AUXM, REC, MIXED, false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order) {
+    trace_body<false, AUXM, REC, MIXED, false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order);
 }
 template <int AUXM, bool REC, bool MIXED, bool DET>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
 void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
-                 uint32_t tiles_y, uint32_t btiles_x) {
-    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x);
+                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order) {
+    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order);
 }
 
 // Closing kernels of the deterministic mode: fixed point -> fp32, added to the caller's (zero-filled) tensors.
@@ -1645,14 +1648,60 @@ __global__ void k_det_finish_weights(const DstParams p) {
     }
 }
 
+// Sort key of a ray of a ray list, so that the 64 rays of a wave run side by side: the cell of the origin on a
+// 32^3 grid over the scene (15 bits), then the direction as a Morton code of its octahedral map (2 x 8 bits).
+// Rays that cannot be keyed (NaN, zero direction) get key 0.
+__global__ void k_ray_keys(const float *__restrict__ ray_o, const float *__restrict__ ray_d, const DstBounds *bounds,
+                           uint32_t *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t n) {
+    const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= n) return;
+    const float ext = __uint_as_float(bounds->max_abs);
+    const float inv = ext > 0.f ? 16.0f / ext : 0.f;
+    uint32_t cell = 0u, dir = 0u;
+    float d[3], l1 = 0.f;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        const float c = fminf(fmaxf(ray_o[3 * (size_t)r + a] * inv + 16.0f, 0.f), 31.f);   // NaN -> 0
+        cell = (cell << 5) | (uint32_t)c;
+        d[a] = ray_d[3 * (size_t)r + a];
+        l1 += fabsf(d[a]);
+    }
+    if (l1 > 0.f && l1 < INFINITY) {
+        float u = d[0] / l1, v = d[1] / l1;
+        if (d[2] < 0.f) {   // fold the lower hemisphere over the square's corners
+            const float fu = (1.f - fabsf(v)) * (u >= 0.f ? 1.f : -1.f), fv = (1.f - fabsf(u)) * (v >= 0.f ? 1.f : -1.f);
+            u = fu;
+            v = fv;
+        }
+        uint32_t qu = (uint32_t)fminf(fmaxf((u * 0.5f + 0.5f) * 256.f, 0.f), 255.f);
+        uint32_t qv = (uint32_t)fminf(fmaxf((v * 0.5f + 0.5f) * 256.f, 0.f), 255.f);
+        auto spread8 = [](uint32_t x) {
+            x = (x | (x << 4)) & 0x0F0Fu;
+            x = (x | (x << 2)) & 0x3333u;
+            x = (x | (x << 1)) & 0x5555u;
+            return x;
+        };
+        dir = (spread8(qu) << 1) | spread8(qv);
+    }
+    keys[r] = (cell << 16) | dir;
+    vals[r] = r;
+}
+
 struct TileGrid {
     int tw_log2, th_log2;
     uint32_t tiles_x, tiles_y, btiles_x, btiles_y;
 };
 
-// 8x8 pixel tiles per wave, 2x2 tiles per block; thin grids (H < 8, e.g. (1,N,3) ray lists) get wider, flatter tiles.
+// 8x8 pixel tiles per wave, 2x2 tiles per block.  A thin grid (H < 8: a (B,N,3) ray list) is one flat list of
+// H*W rays in tiles of 1x64, traced in a coherent order of its own (k_ray_keys).
+constexpr int kThinRows = 8;
+constexpr uint32_t kOrderMinRays = 2048;   // shorter lists are traced as they come
 TileGrid tile_grid(int H, int W) {
     TileGrid t;
+    if (H < kThinRows) {
+        W = H * W;
+        H = 1;
+    }
     t.th_log2 = 3;
     while (t.th_log2 > 0 && (1 << t.th_log2) > H) --t.th_log2;
     t.tw_log2 = 6 - t.th_log2;
@@ -1664,7 +1713,7 @@ TileGrid tile_grid(int H, int W) {
 }
 
 template <bool BWD, bool REC>
-void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipStream_t stream) {
+void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, const uint32_t *ray_order, hipStream_t stream) {
     const uint32_t n_blocks = t.btiles_x * t.btiles_y;
     dim3 grid(n_blocks), block(kWavesPerBlock * DST_WAVE);
     if (!BWD && kFwdWavesPerBlock == 1) {
@@ -1679,13 +1728,13 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, hipS
     do {                                                                                                           \
         if (BWD && det)                                                                                            \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, true>), grid, block, 0, stream, p, acc,      \
-                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                            \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                 \
         else if (BWD)                                                                                              \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, false>), grid, block, 0, stream, p, acc,     \
-                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                            \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                 \
         else                                                                                                       \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED>), grid, block, 0, stream, p, acc, t.tw_log2,          \
-                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x);                                       \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                            \
     } while (0)
 #define DST_LAUNCH(AUX)                                                                                            \
     do {                                                                                                           \
@@ -1723,8 +1772,40 @@ uint64_t dst_hit_record_layout(int32_t H, int32_t W, int32_t mtd_alloc, uint32_t
     return header + (uint64_t)blocks * kRecBlockWords;
 }
 
-int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream) {
-    if (p.H <= 0 || p.W <= 0) return DST_OK;  // empty ray grid: nothing to do
+int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStream_t stream) {
+    if (p_in.H <= 0 || p_in.W <= 0) return DST_OK;  // empty ray grid: nothing to do
+    DstParams p = p_in;
+    const uint32_t *ray_order = nullptr;
+    if (p.H < kThinRows) {
+        // a ray list: flat, and (when it is long enough to matter) in an order that puts similar rays in one wave.
+        // Forward and backward derive the same order from the same rays, so a hit record stays valid.
+        if ((uint64_t)p.H * p.W > 0x7FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
+        p.W = p.H * p.W;
+        p.H = 1;
+        const uint32_t n = (uint32_t)p.W;
+        if (n >= kOrderMinRays) {
+            if (n > ctx->ray_capacity) {
+                for (int k = 0; k < 2; ++k) {
+                    if (ctx->ray_keys[k]) (void)hipFree(ctx->ray_keys[k]);
+                    if (ctx->ray_vals[k]) (void)hipFree(ctx->ray_vals[k]);
+                    ctx->ray_keys[k] = ctx->ray_vals[k] = nullptr;
+                }
+                if (ctx->ray_hist) (void)hipFree(ctx->ray_hist);
+                ctx->ray_hist = nullptr;
+                ctx->ray_capacity = 0;
+                for (int k = 0; k < 2; ++k) {
+                    DST_HIP(ctx, hipMalloc((void **)&ctx->ray_keys[k], sizeof(uint32_t) * n));
+                    DST_HIP(ctx, hipMalloc((void **)&ctx->ray_vals[k], sizeof(uint32_t) * n));
+                }
+                DST_HIP(ctx, hipMalloc((void **)&ctx->ray_hist, sizeof(uint32_t) * dst_sort_hist_elems(n)));
+                ctx->ray_capacity = n;
+            }
+            hipLaunchKernelGGL(k_ray_keys, dim3((n + 255u) / 256u), dim3(256), 0, stream, p.ray_o, p.ray_d, ctx->bounds,
+                               ctx->ray_keys[0], ctx->ray_vals[0], n);
+            dst_sort_pairs(ctx->ray_keys, ctx->ray_vals, ctx->ray_hist, n, stream);
+            ray_order = ctx->ray_vals[0];
+        }
+    }
     const TileGrid t = tile_grid(p.H, p.W);
     if ((uint64_t)t.tiles_x * t.tiles_y > 0x3FFFFFFFull) return dst_fail(ctx, DST_E_INVALID, "ray grid too large");
     DstAccelView acc;
@@ -1737,8 +1818,8 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
     const bool rec = p.hit_record != nullptr;
     const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
     if (backward) {
-        if (rec) launch<true, true>(p, acc, t, stream);   // does the work if the record is complete,
-        launch<true, false>(p, acc, t, stream);           // else this one does (it returns at once otherwise)
+        if (rec) launch<true, true>(p, acc, t, ray_order, stream);   // does the work if the record is complete,
+        launch<true, false>(p, acc, t, ray_order, stream);           // else this one does (it returns at once otherwise)
         if (det) {
             const dim3 grid(2048), block(256);
             if (p.aux <= 2) hipLaunchKernelGGL(k_det_finish_grads<2>, grid, block, 0, stream, p);
@@ -1746,8 +1827,8 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_
             else hipLaunchKernelGGL(k_det_finish_grads<8>, grid, block, 0, stream, p);
         }
     } else {
-        if (rec) launch<false, true>(p, acc, t, stream);
-        else launch<false, false>(p, acc, t, stream);
+        if (rec) launch<false, true>(p, acc, t, ray_order, stream);
+        else launch<false, false>(p, acc, t, ray_order, stream);
         if (det && p.training && p.a_weights != nullptr)
             hipLaunchKernelGGL(k_det_finish_weights, dim3(1024), dim3(256), 0, stream, p);
     }
