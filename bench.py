@@ -182,11 +182,14 @@ def main():
                 traffic = rec["bytes_per_launch"]
         return {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": traffic,
+                # `traffic` is not measured by this run: it is the FETCH_SIZE + WRITE_SIZE figure of the committed
+                # counter runs of the same command (profiles/), which goes stale when the kernels change
+                "traffic_source": None if traffic is None else "profiles/hbm_traffic.json (rocprofv3 --pmc runs of this command)",
                 "algorithmic_bytes_per_launch": int(a_bytes), "avg_launch_ms": round(ms, 4)}
     aux_max = 2 if aux_out <= 2 else (4 if aux_out <= 4 else 8)
     mixed = "true" if (depth > 0 or H < 8) else "false"   # kernels with the per-lane walk built in
     per_kernel = {"forward": roofline_of("forward", "k_trace_fwd<%d,true,%s>" % (aux_max, mixed), A_fwd, fwd_ms),
-                  "backward": roofline_of("backward", "k_trace_bwd<%d,true,false>" % aux_max, A_bwd, bwd_ms)}
+                  "backward": roofline_of("backward", "k_trace_bwd<%d,true,false,false>" % aux_max, A_bwd, bwd_ms)}
     # the dominant kernel is the slower one (the two are within a few per cent of each other on this workload,
     # so both are reported under `roofline_kernels`)
     roofline = per_kernel["backward" if bwd_ms >= fwd_ms else "forward"]
