@@ -599,12 +599,14 @@ __device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v);
 #endif
 constexpr uint32_t kEmptyKey = 0xFFFFFFFFu;
 constexpr int kMaxProbe = 8;
-// row columns: colour 0-2, opacity 3, scales 4-5, rotation 6-9, mean 10-12, densification mean 13-15,
-// aux 16..16+AUXM-1, then SH coefficient j channel c at 16+AUXM+3j+c
-constexpr int kColColor = 0, kColOpac = 3, kColScale = 4, kColRot = 6, kColMean = 10, kColGrad = 13, kColAux = 16;
+// row columns: colour 0-2, opacity 3, scales 4-5, rotation 6-9, mean 10-12, densification mean 13-15, SH coefficient
+// j channel c at 16+3j+c (16..63), aux 64..64+AUXM-1.  The auxiliary channels come last so that a scene without
+// them (the usual one) fills exactly four 16-column tiles of the group reduction and skips the fifth.
+constexpr int kColColor = 0, kColOpac = 3, kColScale = 4, kColRot = 6, kColMean = 10, kColGrad = 13, kColSh = 16,
+              kColAux = 64;
 template <int AUXM> struct RowLayout {
-    static constexpr int sh0 = kColAux + AUXM;
-    static constexpr int cols = sh0 + 48;
+    static constexpr int sh0 = kColSh;
+    static constexpr int cols = kColAux + AUXM;
     static constexpr int stride = cols | 1;     // odd: rows spread over all LDS banks
     // rows of the block's table: with more auxiliary channels the rows are longer, and three blocks must fit a CU
     static constexpr int rows_log2 = AUXM <= 2 ? DST_TABLE_ROWS_LOG2 : DST_TABLE_ROWS_LOG2 - 1;
@@ -622,7 +624,7 @@ template <int AUXM, bool DET> struct TableRows {
 // columns (scale, rotation, mean, densification: range +-6.7e7), 2^-40 for the others and for the blending
 // weights (+-4.2e6); a value outside the range saturates.
 constexpr int kDetShiftGeo = 36, kDetShiftOther = 40;
-__device__ __forceinline__ int det_shift(int col) { return (col >= kColScale && col < kColAux) ? kDetShiftGeo : kDetShiftOther; }
+__device__ __forceinline__ int det_shift(int col) { return (col >= kColScale && col < kColSh) ? kDetShiftGeo : kDetShiftOther; }
 __device__ __forceinline__ long long to_fixed(float v, int shift) {
     float x = __builtin_ldexpf(v, shift);                       // exact scaling
     x = __builtin_fminf(__builtin_fmaxf(x, -4.6e18f), 4.6e18f);   // |x| < 2^62; NaN becomes a bound
@@ -638,12 +640,12 @@ __device__ __forceinline__ float *grad_address(const DstParams &p, uint32_t g, i
     if (col < kColRot) return p.dL_dscales + 2 * (size_t)g + (col - kColScale);
     if (col < kColMean) return p.dL_drotations + 4 * (size_t)g + (col - kColRot);
     if (col < kColGrad) return p.dL_dmeans3D + 3 * (size_t)g + (col - kColMean);
-    if (col < kColAux) return p.dL_dgrads3D + 3 * (size_t)g + (col - kColGrad);
-    if (col < RowLayout<AUXM>::sh0) {
+    if (col < kColSh) return p.dL_dgrads3D + 3 * (size_t)g + (col - kColGrad);
+    if (col >= kColAux) {
         const int ch = col - kColAux;
         return (p.others_precomp != nullptr && ch < p.aux) ? p.dL_dothers + (size_t)p.aux * g + ch : nullptr;
     }
-    const int k = col - RowLayout<AUXM>::sh0;   // 3j + c
+    const int k = col - kColSh;   // 3j + c
     return (p.colors_precomp == nullptr && k < 3 * p.M) ? p.dL_dshs + (size_t)g * p.M * 3 + k : nullptr;
 }
 
@@ -827,7 +829,12 @@ struct BounceAcc {
 
 // The SH colour's derivative with respect to the direction it was evaluated for, contracted with the colour
 // gradient gc (backward.cu:100-165).
-struct LastShHit { int g; F3 gc; bool any; };
+struct LastShHit {
+    int g; F3 gc; bool any;
+#ifdef DST_STATS
+    unsigned long long t0, t_alg, t_sh;
+#endif
+};
 __device__ __forceinline__ F3 sh_direction_gradient(int deg, const float *__restrict__ sh, F3 rd, F3 gc) {
 #pragma clang fp contract(fast)
     auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
@@ -956,6 +963,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
                           w_ * (gR[0].y - gR[1].x));
         g_rot[0] = r0; g_rot[1] = r1; g_rot[2] = r2; g_rot[3] = r3;
     }
+    STAT(last.t_alg += __builtin_readcyclecounter() - last.t0; last.t0 = __builtin_readcyclecounter();)
     // the table columns, in ascending order
     sink.add(kColColor + 0, g_col[0]); sink.add(kColColor + 1, g_col[1]); sink.add(kColColor + 2, g_col[2]);
     sink.add(kColOpac, g_alpha * G * pc);
@@ -965,10 +973,9 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     sink.add(kColMean + 0, g_mean.x); sink.add(kColMean + 1, g_mean.y); sink.add(kColMean + 2, g_mean.z);
     const float hd = 0.5f * dpt;
     sink.add(kColGrad + 0, g_mean.x * hd); sink.add(kColGrad + 1, g_mean.y * hd); sink.add(kColGrad + 2, g_mean.z * hd);
-#pragma unroll
-    for (int ch = 0; ch < AUXM; ++ch) sink.add(kColAux + ch, g_aux_w[ch]);
-    if (p.colors_precomp != nullptr) sink.finish(RowLayout<AUXM>::sh0);
+    // (the first tile, columns 0..15, has just been reduced: its last column triggers that)
 
+    STAT(last.t_sh += __builtin_readcyclecounter() - last.t0;)   // first tile done
     if (p.colors_precomp == nullptr) {
         // SH backward (backward.cu:68-166); the direction gradient REPLACES the ray's (backward.cu:165)
         const int deg = p.D;
@@ -1006,8 +1013,7 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
             }
         }
 #pragma unroll
-        for (int j = 0; j < 16; ++j) put(j, basis[j]);
-        sink.finish(RowLayout<AUXM>::cols);
+        for (int j = 0; j < 16; ++j) put(j, basis[j]);   // columns 16..63: three full tiles
         // The reference overwrites the ray-direction gradient with the SH term at every hit (backward.cu:165), so
         // only the last composited hit's term survives: remember it, walk_bounce computes it once per bounce.
         if (did) {
@@ -1015,6 +1021,11 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
             last.gc = gc;
             last.any = true;
         }
+    }
+    if (p.others_precomp != nullptr) {   // the fifth tile only where there are auxiliary channels
+#pragma unroll
+        for (int ch = 0; ch < AUXM; ++ch) sink.add(kColAux + ch, g_aux_w[ch]);
+        sink.finish(RowLayout<AUXM>::cols);
     }
 }
 
@@ -1119,6 +1130,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     bool live = lane_on;
     KBuf buf;
     LastShHit last_sh = {0, f3(0, 0, 0), false};
+    STAT(last_sh.t_alg = 0; last_sh.t_sh = 0;)
     // kernels built without the per-lane walk (MIXED false) take every wave as a packet
     const bool as_packet = (!MIXED || (REC && BWD)) ? true : rays_run_together(ro, rd, lane_on, max_abs);
     uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
@@ -1261,7 +1273,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                     for (int ch = 0; ch < AUXM; ++ch)
                         if (ch < p.aux) run.O[ch] += w * p.others_precomp[(size_t)p.aux * g + ch];
                 }
-                if (!BWD && (p.flags & DST_FLAG_DISTORTION)) {
+                if (!BWD && DET && (p.flags & DST_FLAG_DISTORTION)) {
                     // depth distortion of 2DGS with its running moments (x = distortion, y = M1, z = M2); the
                     // reference declares the three and leaves the computation open (forward.cu:286)
                     const float A_before = 1 - Tp;
@@ -1283,7 +1295,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             } while (false);
             if (REC && BWD) fetch_geometry(want_next);
             if (!BWD && p.training && p.a_weights != nullptr)
-                wave_add_grouped(p.a_weights, (p.flags & DST_FLAG_DETERMINISTIC) ? p.det_workspace : nullptr, did, (uint32_t)g, w);
+                wave_add_grouped(p.a_weights, (DET && (p.flags & DST_FLAG_DETERMINISTIC)) ? p.det_workspace : nullptr, did,
+                                 (uint32_t)g, w);
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
             if (BWD && wave_ballot(did) != 0ull) {
                 GradSink<AUXM, DET> sink;
@@ -1292,9 +1305,10 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 sink.stage = stage;
                 sink.did = did;
                 sink.g = (uint32_t)g;
-                sink.limit = (p.colors_precomp == nullptr) ? RowLayout<AUXM>::cols : RowLayout<AUXM>::sh0;
+                sink.limit = RowLayout<AUXM>::cols;   // dead columns (no SH, no aux) are never staged
                 STAT(unsigned long long d0 = __builtin_readcyclecounter();)
                 sink.plan(tab_keys);
+                STAT(last_sh.t0 = __builtin_readcyclecounter();)
                 STAT(unsigned long long d1 = __builtin_readcyclecounter(); ws.t_plan += d1 - d0; ws.steps++;
                      ws.nodes += __popcll(wave_ballot(did && sink.own_slot < 0)); ws.leaves += __popcll(wave_ballot(sink.stray));
                      ws.leaf_any += __popcll(wave_ballot(did));)
@@ -1325,6 +1339,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         }
     }
+    STAT(if (BWD) { ws.nodes = last_sh.t_alg; ws.leaves = last_sh.t_sh; })
     if (BWD && p.colors_precomp == nullptr && last_sh.any)
         g_rd = sh_direction_gradient(p.D, p.shs + (size_t)last_sh.g * p.M * 3, rd, last_sh.gc);
     run.T = Tp;
@@ -1412,7 +1427,8 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     const bool inside = wave_on && py < (uint32_t)p.H && px < (uint32_t)p.W;
     // ray lists are traced in a coherent order (see k_ray_keys): position in that order -> ray number
     const size_t pos = inside ? ((size_t)py * p.W + px) : 0;
-    const size_t r = (ray_order != nullptr && inside) ? (size_t)ray_order[pos] : pos;
+    // (forward: ray lists always run the MIXED kernels, so the image kernels need not look at the order)
+    const size_t r = ((MIXED || BWD) && ray_order != nullptr && inside) ? (size_t)ray_order[pos] : pos;
     const float max_abs = __uint_as_float(acc.bounds->max_abs);
     const int MID = 14 + p.aux, AUXO = 11, RGBO = 11 + p.aux;
     const int slots = p.mtd_alloc + 1, mtd = p.max_trace_depth;
@@ -1438,7 +1454,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             F3 dist_acc = f3(0, 0, 0);
-            walk_bounce<false, AUXM, REC, MIXED, false>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i, dist_acc WS_ARG);
+            walk_bounce<false, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i, dist_acc WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -1614,11 +1630,13 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
 #ifndef DST_BWD_WAVES
 #define DST_BWD_WAVES 3
 #endif
-template <int AUXM, bool REC, bool MIXED>
+// EXTRAS: the rarely used forward options (DstParams.flags: fixed-point blending weights, distortion output) live in
+// a kernel of their own, so that the usual one does not carry their registers.
+template <int AUXM, bool REC, bool MIXED, bool EXTRAS>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order) {
-    trace_body<false, AUXM, REC, MIXED, false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order);
+    trace_body<false, AUXM, REC, MIXED, EXTRAS>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order);
 }
 template <int AUXM, bool REC, bool MIXED, bool DET>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
@@ -1732,8 +1750,11 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
         else if (BWD)                                                                                              \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, false>), grid, block, 0, stream, p, acc,     \
                                t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                 \
+        else if (p.flags != 0u)                                                                                    \
+            hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, true>), grid, block, 0, stream, p, acc, t.tw_log2,    \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                            \
         else                                                                                                       \
-            hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED>), grid, block, 0, stream, p, acc, t.tw_log2,          \
+            hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, false>), grid, block, 0, stream, p, acc, t.tw_log2,   \
                                t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                            \
     } while (0)
 #define DST_LAUNCH(AUX)                                                                                            \
