@@ -188,7 +188,7 @@ def main():
                 "algorithmic_bytes_per_launch": int(a_bytes), "avg_launch_ms": round(ms, 4)}
     aux_max = 2 if aux_out <= 2 else (4 if aux_out <= 4 else 8)
     mixed = "true" if (depth > 0 or H < 8) else "false"   # kernels with the per-lane walk built in
-    per_kernel = {"forward": roofline_of("forward", "k_trace_fwd<%d,true,%s>" % (aux_max, mixed), A_fwd, fwd_ms),
+    per_kernel = {"forward": roofline_of("forward", "k_trace_fwd<%d,true,%s,false>" % (aux_max, mixed), A_fwd, fwd_ms),
                   "backward": roofline_of("backward", "k_trace_bwd<%d,true,false,false>" % aux_max, A_bwd, bwd_ms)}
     # the dominant kernel is the slower one (the two are within a few per cent of each other on this workload,
     # so both are reported under `roofline_kernels`)

@@ -1310,7 +1310,6 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 sink.plan(tab_keys);
                 STAT(last_sh.t0 = __builtin_readcyclecounter();)
                 STAT(unsigned long long d1 = __builtin_readcyclecounter(); ws.t_plan += d1 - d0; ws.steps++;
-                     ws.nodes += __popcll(wave_ballot(did && sink.own_slot < 0)); ws.leaves += __popcll(wave_ballot(sink.stray));
                      ws.leaf_any += __popcll(wave_ballot(did));)
                 hit_backward<AUXM, DET>(p, in, run, did ? g : 0, e_i, Tp_hit, alpha, G, w, dpt_hit, xyz, R, u, v, sx, sy, mean,
                                    q0, q1, q2, q3, opac, nsign, normal, col, neg, ro, rd, sh, g_ro, g_rd, sink, did, last_sh);
@@ -1339,7 +1338,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         }
     }
-    STAT(if (BWD) { ws.nodes = last_sh.t_alg; ws.leaves = last_sh.t_sh; })
+    STAT(if (BWD) { ws.nodes += last_sh.t_alg; ws.leaves += last_sh.t_sh; })
     if (BWD && p.colors_precomp == nullptr && last_sh.any)
         g_rd = sh_direction_gradient(p.D, p.shs + (size_t)last_sh.g * p.M * 3, rd, last_sh.gc);
     run.T = Tp;
