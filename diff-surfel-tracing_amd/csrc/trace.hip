@@ -450,8 +450,13 @@ typedef __attribute__((address_space(3))) uint32_t *lds_u32;
 // `shelf`: optional LDS for the first kLaneShelf stack entries of every lane ([entry][lane], conflict-free);
 // deeper entries, or all of them without a shelf, live in private memory.
 constexpr int kLaneShelf = 32;
-__device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, const RaySlab &slab, F3 o, F3 d,
-                                                    bool active, KBuf &buf, uint32_t &cnt, uint32_t *shelf) {
+struct LaneWalkAccel { const DstLeaf *leaves; const DstWideNode *wide; uint32_t n_leaves, root; };   // by value: registers
+__device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc, const RaySlab &slab, F3 o, F3 d,
+                                                    bool active, KBuf &buf_mem, uint32_t &cnt_mem, uint32_t *shelf) {
+    // The caller's buffer is in memory (its address crosses the call): work on a register copy and store it once
+    // at the end.  Left in memory, every leaf test re-read its 128 bytes per lane and every admission re-wrote them.
+    KBuf buf = buf_mem;
+    uint32_t cnt = cnt_mem;
     RaySlabFast fs;
     fs.ix = slab.ix; fs.iy = slab.iy; fs.iz = slab.iz;
     fs.cnx = slab.nx - slab.wx; fs.cny = slab.ny - slab.wy; fs.cnz = slab.nz - slab.wz;
@@ -528,6 +533,8 @@ __device__ __attribute__((noinline)) void lane_walk(const DstAccelView &acc, con
         }
         ref = (--budget == 0u) ? kWalkDone : next;
     }
+    buf_mem = buf;
+    cnt_mem = cnt;
 }
 
 // Packet or per-lane walk for the rays of this wave?  A packet pays off when the rays run side by side: every
@@ -567,7 +574,8 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
         uint32_t n = cnt;
         // forward kernels (one wave per workgroup, no other LDS) give the walk an LDS shelf for its stacks
         __shared__ uint32_t s_shelf[SHELF ? kFwdWavesPerBlock * kLaneShelf * DST_WAVE : 1];
-        lane_walk(acc, slab, o, d, active, mine, n,
+        const LaneWalkAccel view = {acc.leaves, acc.wide, acc.n_leaves, acc.root};
+        lane_walk(view, slab, o, d, active, mine, n,
                   SHELF ? s_shelf + (threadIdx.x / DST_WAVE) * (kLaneShelf * DST_WAVE) : nullptr);
         buf = mine;
         cnt = n;
@@ -1407,7 +1415,8 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     // eight times more distinct BVH data in the shared last-level cache), and compact neighbouring patches of 2x4
     // to 8x16 blocks per XCD inside super-tiles (+1 % to +13 %, more with larger patches).
     const uint32_t bx = bid % btiles_x, by = bid / btiles_x;
-    if (2u * by >= tiles_y) return;   // padding of the forward grid (whole blocks)
+    const bool flat = th_log2 == 0;   // a ray list: tiles of 1x64 rays, a block = four consecutive tiles
+    if (flat ? by >= 1u : 2u * by >= tiles_y) return;   // padding of the forward grid (whole blocks)
     RecView rv = {nullptr, nullptr, nullptr, 0u};
     if (REC) {
         const uint32_t n_waves = btiles_x * ((tiles_y + 1u) / 2u) * kWavesPerBlock, slots_ = (uint32_t)p.mtd_alloc + 1u;
@@ -1417,7 +1426,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         rv.blocks = p.hit_record + 2 + dir_words;
         rv.capacity = p.hit_record_blocks;
     }
-    const uint32_t ty = 2u * by + (wv >> 1), tx = 2u * bx + (wv & 1u);
+    const uint32_t ty = flat ? 0u : 2u * by + (wv >> 1), tx = flat ? 4u * bx + wv : 2u * bx + (wv & 1u);
     const bool wave_on = ty < tiles_y && tx < tiles_x;
     if (!BWD && !wave_on) return;   // the backward kernel keeps every wave for the block-wide flush below
     const uint32_t lane = threadIdx.x % DST_WAVE;
@@ -1724,8 +1733,13 @@ TileGrid tile_grid(int H, int W) {
     t.tw_log2 = 6 - t.th_log2;
     t.tiles_x = ((uint32_t)W + (1u << t.tw_log2) - 1) >> t.tw_log2;
     t.tiles_y = ((uint32_t)H + (1u << t.th_log2) - 1) >> t.th_log2;
-    t.btiles_x = (t.tiles_x + 1) / 2;
-    t.btiles_y = (t.tiles_y + 1) / 2;
+    if (t.th_log2 == 0) {   // a list: a block is four consecutive tiles
+        t.btiles_x = (t.tiles_x + 3) / 4;
+        t.btiles_y = 1;
+    } else {
+        t.btiles_x = (t.tiles_x + 1) / 2;
+        t.btiles_y = (t.tiles_y + 1) / 2;
+    }
     return t;
 }
 
