@@ -642,7 +642,7 @@ __device__ __forceinline__ float from_fixed(long long q, int shift) { return (fl
 
 // Address in the caller's gradient tensors of column `col` of surfel g (nullptr: nothing to write).
 template <int AUXM>
-__device__ __forceinline__ float *grad_address(const DstParams &p, uint32_t g, int col) {
+__device__ __forceinline__ float *tensor_address(const DstParams &p, uint32_t g, int col) {
     if (col < kColOpac) return p.dL_dcolors + 3 * (size_t)g + col;
     if (col < kColScale) return p.dL_dopacities + g;
     if (col < kColRot) return p.dL_dscales + 2 * (size_t)g + (col - kColScale);
@@ -655,6 +655,20 @@ __device__ __forceinline__ float *grad_address(const DstParams &p, uint32_t g, i
     }
     const int k = col - kColSh;   // 3j + c
     return (p.colors_precomp == nullptr && k < 3 * p.M) ? p.dL_dshs + (size_t)g * p.M * 3 + k : nullptr;
+}
+// Is column `col` in use?  (no auxiliary input: no aux columns; colours given: no SH columns; SH degree < 3: fewer)
+template <int AUXM>
+__device__ __forceinline__ bool column_live(const DstParams &p, int col) {
+    if (col < kColSh) return true;
+    if (col >= kColAux) return p.others_precomp != nullptr && col - kColAux < p.aux;
+    return p.colors_precomp == nullptr && col - kColSh < 3 * p.M;
+}
+// Where the kernels add column `col` of surfel g: the row of g in the caller's gradient rows if there are any
+// (all columns of a surfel side by side; a closing kernel adds the rows to the tensors), else the tensors.
+template <int AUXM>
+__device__ __forceinline__ float *grad_address(const DstParams &p, uint32_t g, int col) {
+    if (p.grad_rows == nullptr) return tensor_address<AUXM>(p, g, col);
+    return column_live<AUXM>(p, col) ? p.grad_rows + (size_t)g * RowLayout<AUXM>::cols + col : nullptr;
 }
 
 // Sum of v over the 64 lanes; every lane must be active.
@@ -746,6 +760,7 @@ struct GradSink {
     int out_slot;        // table row of group lane%16, -1: write through to global memory
     uint32_t out_g;      // surfel of group lane%16
     int limit;           // columns in use
+    uint64_t wt;         // wave-uniform: lanes whose surfel has no table row (their values go to global memory)
 
     // Wave-uniform; every lane of the wave must be active.
     __device__ __forceinline__ void plan(uint32_t *keys) {
@@ -775,22 +790,55 @@ struct GradSink {
         own_slot = did ? table_slot<TableRows<AUXM, DET>::rows_log2>(keys, g) : -1;
         out_slot = __builtin_amdgcn_ds_bpermute((int)(leader << 2), own_slot);
         out_g = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(leader << 2), (int)g);
+        // (deterministic mode: a group's sum must be rounded to fixed point as one number whether or not it finds
+        // a table row, which depends on timing; so only the lanes outside the groups take this route there)
+        wt = wave_ballot(did && own_slot < 0 && (!DET || stray));
     }
 
-    __device__ __forceinline__ void put(int slot, uint32_t surfel, int col, float v) const {
+    __device__ __forceinline__ void put_global(uint32_t surfel, int col, float v) const {
         if (DET) {
-            const long long q = to_fixed(v, det_shift(col));
-            if (slot >= 0)
-                __hip_atomic_fetch_add(reinterpret_cast<long long *>(rows) + (size_t)slot * RowLayout<AUXM>::stride + col, q,
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            else if (grad_address<AUXM>(*p, surfel, col) != nullptr)
-                atomicAdd(p->det_workspace + (size_t)surfel * RowLayout<AUXM>::cols + col, (unsigned long long)q);
-        } else if (slot >= 0) {
-            __hip_atomic_fetch_add(rows + (size_t)slot * RowLayout<AUXM>::stride + col, v, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (column_live<AUXM>(*p, col))
+                atomicAdd(p->det_workspace + (size_t)surfel * RowLayout<AUXM>::cols + col,
+                          (unsigned long long)to_fixed(v, det_shift(col)));
         } else {
             float *dst = grad_address<AUXM>(*p, surfel, col);
             if (dst != nullptr) aadd(dst, v);
+        }
+    }
+
+    // Add v to column `col` of table row `slot` (>= 0).
+    __device__ __forceinline__ void put(int slot, int col, float v) const {
+        if (DET)
+            __hip_atomic_fetch_add(reinterpret_cast<long long *>(rows) + (size_t)slot * RowLayout<AUXM>::stride + col,
+                                   to_fixed(v, det_shift(col)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else
+            __hip_atomic_fetch_add(rows + (size_t)slot * RowLayout<AUXM>::stride + col, v, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+
+    // The staged tile's values of the lanes in `wt`, added to global memory.  Sixteen lanes take the sixteen
+    // columns of one such lane's hit, so that one instruction adds to four runs of consecutive addresses (four hits)
+    // instead of to one address in each of up to 64 surfels' rows: the memory system works on whole cache lines.
+    __device__ __forceinline__ void write_through(int tile) const {
+        const uint32_t lane = __lane_id();
+        const int c = (int)(lane & 15u), k = (int)(lane >> 4);
+        const int col = tile * kStageCols + c;
+        uint64_t m = wt;
+#pragma unroll 1
+        while (m != 0ull) {
+            int h = -1;   // quarter k of the wave takes the k-th of the next four hits
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (m != 0ull) {
+                    const int hq = __builtin_ctzll(m);
+                    m &= m - 1ull;
+                    if (k == q) h = hq;
+                }
+            }
+            const int src = h < 0 ? 0 : h;
+            const uint32_t gh = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)g);   // every lane is active here
+            const float v = stage[c * kStageStride + src];
+            if (h >= 0 && col < limit && v != 0.f) put_global(gh, col, v);
         }
     }
 
@@ -806,8 +854,12 @@ struct GradSink {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int col = tile * kStageCols + 4 * (int)(lane >> 4) + r;
-            if (out_on && col < limit && acc[r] != 0.f) put(out_slot, out_g, col, acc[r]);
+            if (out_on && col < limit && acc[r] != 0.f) {
+                if (out_slot >= 0) put(out_slot, col, acc[r]);
+                else if (DET) put_global(out_g, col, acc[r]);
+            }
         }
+        if (wt != 0ull) write_through(tile);   // groups and further lanes without a table row
     }
 
     // Wave-uniform calls in ascending column order (every lane reaches them); `col` is a constant after
@@ -815,7 +867,7 @@ struct GradSink {
     __device__ __forceinline__ void add(int col, float v) const {
         stage[(col & (kStageCols - 1)) * kStageStride + __lane_id()] = did ? v : 0.f;
         if (any_stray) {   // rare: more than sixteen surfels in one step
-            if (stray && col < limit) put(own_slot, g, col, v);
+            if (stray && own_slot >= 0 && col < limit) put(own_slot, col, v);
         }
         if ((col & (kStageCols - 1)) == kStageCols - 1) flush(col / kStageCols);
     }
@@ -1042,8 +1094,11 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
 //   [0] blocks requested so far (the forward kernel counts on past the capacity, which is how overflow shows)
 //   [1] chains that a replay found broken (stays 0 for a record written by a forward trace with a zeroed header)
 //   [2 ...) directory: one uint32 per (wave, bounce slot) = 1 + first block of that wave's bounce, 0 = none
-//   then `capacity` blocks of kRecBlockWords words: 16x64 entries ([slot][lane]), 64 uint32 counts, next+1.
-constexpr uint32_t kRecBlockWords = kChunk * DST_WAVE + DST_WAVE / 2 + 8;
+//   then `capacity` blocks of kRecBlockWords words: 16x64 entries ([slot][lane]), 64 uint32 counts, next+1, and
+//   the colour of every composited hit as the forward evaluated it ([slot][channel][lane] floats; a channel clamped
+//   at zero is stored as -0): the replay then neither gathers nor evaluates the 48 SH coefficients per hit again.
+constexpr uint32_t kRecColourWord = kChunk * DST_WAVE + DST_WAVE / 2 + 8;   // first word of the colours
+constexpr uint32_t kRecBlockWords = kRecColourWord + kChunk * 3 * DST_WAVE / 2;
 struct RecView {
     uint64_t *base;      // nullptr: not recording / not replaying
     uint64_t *blocks;    // first block
@@ -1052,12 +1107,13 @@ struct RecView {
 };
 
 // Forward: append one chunk of this wave to the record.  `prev` is the wave's previous block in this bounce.
-__device__ __forceinline__ void rec_store(const RecView &rv, int bounce, uint32_t &prev, const KBuf &buf, uint32_t cnt) {
+// Returns where the chunk's colours go (nullptr: the record is full).
+__device__ __forceinline__ float *rec_store(const RecView &rv, int bounce, uint32_t &prev, const KBuf &buf, uint32_t cnt) {
     const uint32_t lane = __lane_id();
     uint32_t blk = 0;
     if (lane == 0) blk = (uint32_t)atomicAdd((unsigned long long *)rv.base, 1ull);
     blk = __builtin_amdgcn_readfirstlane(blk);
-    if (blk >= rv.capacity) return;   // too small: the host sees the count and the backward pass re-traces
+    if (blk >= rv.capacity) return nullptr;   // too small: the host sees the count and the backward pass re-traces
     uint64_t *b = rv.blocks + (size_t)blk * kRecBlockWords;
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) b[k * DST_WAVE + lane] = buf.e[k];
@@ -1069,6 +1125,7 @@ __device__ __forceinline__ void rec_store(const RecView &rv, int bounce, uint32_
         else reinterpret_cast<uint32_t *>(rv.blocks + (size_t)prev * kRecBlockWords + kChunk * DST_WAVE)[DST_WAVE] = blk + 1u;
     }
     prev = blk;
+    return reinterpret_cast<float *>(b + kRecColourWord);
 }
 
 // Backward: locate the next chunk of this wave's bounce; its entries are then read one slot at a time.
@@ -1098,7 +1155,7 @@ __device__ __forceinline__ void table_flush(const DstParams &p, uint32_t *keys, 
             const long long q = qrows[k];
             if (q == 0) continue;
             qrows[k] = 0;
-            if (grad_address<AUXM>(p, g, col) != nullptr)
+            if (column_live<AUXM>(p, col))
                 atomicAdd(p.det_workspace + (size_t)g * RowLayout<AUXM>::cols + col, (unsigned long long)q);
         } else {
             const float v = rows[k];
@@ -1157,6 +1214,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         // Where the compositing loop below takes its entries from: the recorded block, one slot at a time
         // (backward replay: no buffer registers at all), or the register buffer the traversal just filled.
         const uint64_t *rec_block = nullptr;
+        float *rec_colours = nullptr;   // forward with a record: where this chunk's hit colours are kept
         const uint32_t lane_ = __lane_id();
         if (REC && BWD) {
             rec_block = rec_open(rv, rec_pos, cnt);
@@ -1168,7 +1226,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         } else {
             kbuf_reset(buf);
             packet_knn<MIXED, MIXED && !BWD>(acc, max_abs, ot, rd, live, buf, cnt, as_packet WSP);
-            if (REC && !BWD) rec_store(rv, bounce, rec_pos, buf, cnt);
+            if (REC && !BWD) rec_colours = rec_store(rv, bounce, rec_pos, buf, cnt);
         }
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
         int here = 0;
@@ -1264,7 +1322,15 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 if (contrib > kMaxContrib) { stop = true; break; }
                 last_g = g;
                 w = alpha * Tp;
-                if (p.colors_precomp == nullptr) {
+                if (REC && BWD) {   // as the forward trace evaluated it
+                    const float *cs = reinterpret_cast<const float *>(rec_block + kRecColourWord) + it * 3 * DST_WAVE + lane_;
+#pragma unroll
+                    for (int ch = 0; ch < 3; ++ch) {
+                        col[ch] = cs[ch * DST_WAVE];
+                        // -0: clamped (a colour evaluated from SH is never negative; given colours may be)
+                        neg[ch] = p.colors_precomp == nullptr && (__float_as_uint(col[ch]) >> 31) != 0u;
+                    }
+                } else if (p.colors_precomp == nullptr) {
                     sh = p.shs + (size_t)g * p.M * 3;
                     F3 c = sh_color(p.D, sh, rd, neg);
                     col[0] = c.x; col[1] = c.y; col[2] = c.z;
@@ -1272,6 +1338,11 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                     col[0] = p.colors_precomp[3 * (size_t)g];
                     col[1] = p.colors_precomp[3 * (size_t)g + 1];
                     col[2] = p.colors_precomp[3 * (size_t)g + 2];
+                }
+                if (REC && !BWD && rec_colours != nullptr) {
+                    float *cs = rec_colours + it * 3 * DST_WAVE + lane_;
+#pragma unroll
+                    for (int ch = 0; ch < 3; ++ch) cs[ch * DST_WAVE] = neg[ch] ? -0.0f : col[ch];
                 }
                 run.C[0] += w * col[0];
                 run.C[1] += w * col[1];
@@ -1663,8 +1734,22 @@ __global__ void k_det_finish_grads(const DstParams p) {
         if (q == 0) continue;
         const uint32_t g = (uint32_t)(k / cols);
         const int col = (int)(k - (size_t)g * cols);
-        float *dst = grad_address<AUXM>(p, g, col);
+        float *dst = tensor_address<AUXM>(p, g, col);
         if (dst != nullptr) *dst += from_fixed(q, det_shift(col));
+    }
+}
+// Closing kernel of a backward trace with gradient rows: rows -> the caller's tensors.
+template <int AUXM>
+__global__ void k_finish_grad_rows(const DstParams p) {
+    constexpr int cols = RowLayout<AUXM>::cols;
+    const size_t n = (size_t)p.P * cols;
+    for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < n; k += (size_t)gridDim.x * blockDim.x) {
+        const float v = p.grad_rows[k];
+        if (v == 0.f) continue;
+        const uint32_t g = (uint32_t)(k / cols);
+        const int col = (int)(k - (size_t)g * cols);
+        float *dst = tensor_address<AUXM>(p, g, col);
+        if (dst != nullptr) *dst += v;
     }
 }
 __global__ void k_det_finish_weights(const DstParams p) {
@@ -1854,11 +1939,15 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
     if (backward) {
         if (rec) launch<true, true>(p, acc, t, ray_order, stream);   // does the work if the record is complete,
         launch<true, false>(p, acc, t, ray_order, stream);           // else this one does (it returns at once otherwise)
+        const dim3 grid(2048), block(256);
         if (det) {
-            const dim3 grid(2048), block(256);
             if (p.aux <= 2) hipLaunchKernelGGL(k_det_finish_grads<2>, grid, block, 0, stream, p);
             else if (p.aux <= 4) hipLaunchKernelGGL(k_det_finish_grads<4>, grid, block, 0, stream, p);
             else hipLaunchKernelGGL(k_det_finish_grads<8>, grid, block, 0, stream, p);
+        } else if (p.grad_rows != nullptr) {
+            if (p.aux <= 2) hipLaunchKernelGGL(k_finish_grad_rows<2>, grid, block, 0, stream, p);
+            else if (p.aux <= 4) hipLaunchKernelGGL(k_finish_grad_rows<4>, grid, block, 0, stream, p);
+            else hipLaunchKernelGGL(k_finish_grad_rows<8>, grid, block, 0, stream, p);
         }
     } else {
         if (rec) launch<false, true>(p, acc, t, ray_order, stream);

@@ -32,7 +32,7 @@ class DstParams(C.Structure):
                               "others_precomp", "opacities", "scales", "rotations")]
         + [(n, _FP) for n in ("out_rgb", "out_dpt", "out_acc", "out_norm", "out_dist", "out_aux", "mid_val",
                               "a_weights", "counters", "hit_record")]
-        + [("hit_record_blocks", C.c_uint32), ("flags", C.c_uint32), ("det_workspace", _FP)]
+        + [("hit_record_blocks", C.c_uint32), ("flags", C.c_uint32), ("det_workspace", _FP), ("grad_rows", _FP)]
         + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
         + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
                               "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
@@ -195,6 +195,7 @@ class OptiXStateWrapper:
         self.record_max_bytes = 8 << 30     # no record larger than this is made (backward then re-traces)
         self.record_wanted = True           # set by the autograd wrapper for the call that follows
         self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
+        self.gradient_rows = True           # backward sums per-surfel gradients in one row per surfel first (faster)
         self.distortion = False             # True: the dist output carries the 2DGS depth distortion (else zeros)
         self._record_pool = []              # free storages (int64 tensors)
         self._record_fixed = False          # True: only caller-provided storage is used, nothing is allocated
@@ -209,10 +210,13 @@ class OptiXStateWrapper:
         self._record_fixed = storage is not None
 
     def update_record_estimate(self):
-        """Raise the sizing estimate from records whose forward trace has finished; never waits."""
+        """Raise the sizing estimate from records whose forward trace has finished.  Never waits, except in the
+        deterministic mode: whether a backward trace replays a complete record or walks the BVH again changes its
+        gradients in the last bit (the two kernels contract their gradient algebra differently), so there the
+        sequence of record sizes must not depend on timing."""
         still = []
         for rec in self._record_watch:
-            asked = rec.asked()
+            asked = rec.asked(wait=self.deterministic)
             if asked is None:
                 still.append(rec)
             else:
@@ -424,6 +428,10 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
     if getattr(ctx, "deterministic", False):
         det_ws = torch.zeros(load_library().dst_det_workspace_words(P, p.aux, 1), dtype=torch.int64, device=dev)
         p.flags, p.det_workspace = FLAG_DETERMINISTIC, det_ws.data_ptr()
+    elif getattr(ctx, "gradient_rows", True):
+        # the per-surfel gradients are summed in rows of one buffer first (a surfel's columns side by side)
+        det_ws = torch.zeros(load_library().dst_det_workspace_words(P, p.aux, 1), dtype=torch.float32, device=dev)
+        p.grad_rows = det_ws.data_ptr()
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))

@@ -34,13 +34,17 @@ def test_two_runs_are_bit_identical_and_match_the_oracle(oracle, tracer, case):
     ctx = tracer.optix_context
     saved = ctx.record_blocks_per_wave
     tracer.deterministic = True
+    saved_cap = ctx.record_max_bytes
     try:
+        # Runs are compared like with like: all three replay a complete record, or all three walk the BVH again
+        # (the two backward kernels agree to rounding, not to the bit: their gradient algebra may be contracted
+        # differently).
         if case == "record_too_small":
-            ctx.record_blocks_per_wave = 0.01          # backward walks the BVH again instead of replaying
+            ctx.record_max_bytes = 0                   # no record at all: backward walks the BVH again
+        else:
+            _run(tracer, sc, o, d, ug, **kw)           # sizes the record, so that the runs below replay
         runs = []
         for k in range(3):
-            if case == "record_too_small":
-                ctx.record_blocks_per_wave = 0.01
             runs.append(_run(tracer, sc, o, d, ug, **kw))
             torch.cuda.synchronize()
         for out, g in runs[1:]:
@@ -50,6 +54,7 @@ def test_two_runs_are_bit_identical_and_match_the_oracle(oracle, tracer, case):
                     assert np.array_equal(v.view(np.uint32), runs[0][1][k].view(np.uint32)), k
     finally:
         tracer.deterministic = False
+        ctx.record_max_bytes = saved_cap
         ctx.record_blocks_per_wave = max(saved, 6.0)
     out, g = runs[0]
     s = oracle_scene(oracle, sc, o, d, **kw)

@@ -230,6 +230,26 @@ def test_backward_replays_the_forward_hit_record_or_retraces(oracle, tracer):
         ctx.record_blocks_per_wave = max(saved, ctx.record_blocks_per_wave)
 
 
+@pytest.mark.parametrize("case", ["cube_sh3", "room_aux8_depth2"])
+def test_gradients_summed_straight_into_the_tensors(oracle, tracer, case):
+    """The binding hands the backward trace one row of gradient columns per surfel by default (DstParams.grad_rows);
+    a C caller may leave it out, and the kernels then add to the dL_d* tensors directly: same gradients."""
+    ctx = tracer.optix_context
+    assert ctx.gradient_rows
+    ctx.gradient_rows = False
+    try:
+        if case == "cube_sh3":
+            sc = S.scene_cube(P=10000, seed=0)
+            check_case(oracle, tracer, sc, *S.rays_cube(96, 96))
+        else:
+            sc = S.scene_room(P=30000, seed=2, aux=8, half=1.5)
+            sc["others_precomp"][:, 0] = sc["others_precomp"][:, 0] * 0.8 + 0.1
+            o, d = S.pinhole_rays(40, 64, 70.0, (-0.6, -0.3, 0.15), (0.9, 0.45, -0.15))
+            check_case(oracle, tracer, sc, o, d, max_trace_depth=2, specular_threshold=0.1)
+    finally:
+        ctx.gradient_rows = True
+
+
 def test_raw_launcher_calls_without_a_record(oracle, tracer):
     """The four `_C` callables with exactly the reference's positional arguments (24 and 36)."""
     import diff_surfel_tracing._C as binding
