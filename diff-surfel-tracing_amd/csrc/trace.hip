@@ -318,8 +318,9 @@ __device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t fir
                                            , WaveStats &ws
 #endif
 ) {
+    uint32_t q0 = 0;   // count >= 1
 #pragma unroll 1
-    for (uint32_t q0 = 0; q0 < count; q0 += 2) {
+    do {
         const bool two = q0 + 1u < count;
         // the record after the last quad of the structure exists (the array has one spare record)
         uint32_t Q0[16], Q1[16];
@@ -339,7 +340,8 @@ __device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t fir
             load_uniform<19>(&acc.leaves[first + q0 + k], L);
             quad_exact(L, o, d, active, buf, cnt WSP);
         }
-    }
+        q0 += 2;
+    } while (DST_GROUP > 2 && q0 < count);   // groups of at most two quads: one pass, no loop
 }
 
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
@@ -368,13 +370,24 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
     int sp = 0;
     uint32_t ref = acc.root;
     // A well-formed hierarchy is walked in at most one step per node and per leaf group; the cap makes the
-    // loop finite whatever the memory holds.
-    for (uint32_t budget = 2u * acc.n_leaves + 8u; budget != 0u; --budget) {
-        if (ref & DST_LEAF_BIT) {
-            const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
-            if (first + count <= acc.n_leaves) test_group(acc, first, count, rp, o, d, active, buf, cnt WSP);
-        } else {
-            if (ref + 1u >= acc.n_leaves) break;   // not a node of this hierarchy
+    // loops finite whatever the memory holds.  Two loops: the inner one goes down through nodes and never touches
+    // the hit buffer, the outer one tests a leaf group and pops (with one loop around both, the compiler kept two
+    // copies of the buffer's 32 registers and moved them back and forth at every leaf group).
+    constexpr uint32_t kEnd = 0xFFFFFFFFu;   // not a reference: leaf bit set, impossible position
+    uint32_t budget = 2u * acc.n_leaves + 8u;
+    auto pop = [&]() -> uint32_t {
+        if (sp == 0) return kEnd;
+        --sp;
+        const uint32_t a = __builtin_amdgcn_readlane(stack0, sp & 63), b = __builtin_amdgcn_readlane(stack1, sp & 63);
+        return sp < 64 ? a : b;
+    };
+    for (;;) {
+        while ((ref & DST_LEAF_BIT) == 0u) {
+            if (budget == 0u || ref + 1u >= acc.n_leaves) {   // spent, or not a node of this hierarchy
+                ref = kEnd;
+                break;
+            }
+            --budget;
             const char *node = reinterpret_cast<const char *>(&acc.wide[ref]);
             STAT(ws.nodes++;)
             const float tmax = active ? kb_t(buf.e[kChunk - 1]) : -1.0f;
@@ -413,15 +426,16 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                 if ((hit & 2u) && (hit & 1u)) DST_PUSH(tail[1])
 #undef DST_PUSH
                 ref = (hit & 1u) ? tail[0] : ((hit & 2u) ? tail[1] : ((hit & 4u) ? tail[2] : tail[3]));
-                continue;
+            } else {
+                ref = pop();
             }
         }
-        if (sp == 0) break;
-        --sp;
-        {
-            const uint32_t a = __builtin_amdgcn_readlane(stack0, sp & 63), b = __builtin_amdgcn_readlane(stack1, sp & 63);
-            ref = sp < 64 ? a : b;
-        }
+        if (ref == kEnd || budget == 0u) break;
+        --budget;
+        const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
+        if (first + count > acc.n_leaves) break;   // not a leaf group of this hierarchy
+        test_group(acc, first, count, rp, o, d, active, buf, cnt WSP);
+        ref = pop();
     }
 }
 
@@ -602,6 +616,9 @@ __device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v);
 // are first summed in an LDS hash table (one row of columns per surfel, LDS atomics) and written to
 // global memory once per surfel and block when the block ends.  A surfel that finds no free row within a
 // few probes goes straight to global atomics, so the table can never be wrong, only less effective.
+#ifndef DST_TABLE_FLUSH_NUM
+#define DST_TABLE_FLUSH_NUM 6   // the table is emptied between rounds once this many eighths of its rows are in use
+#endif
 #ifndef DST_TABLE_ROWS_LOG2
 #define DST_TABLE_ROWS_LOG2 7
 #endif
@@ -1410,7 +1427,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         } while (false);
         if (BWD) {
             __syncthreads();   // every wave's additions of this round are in the table
-            if (tab_keys[TableRows<AUXM, DET>::rows] > (uint32_t)(3 * TableRows<AUXM, DET>::rows / 4)) {
+            if (tab_keys[TableRows<AUXM, DET>::rows] > (uint32_t)(DST_TABLE_FLUSH_NUM * TableRows<AUXM, DET>::rows / 8)) {
                 table_flush<AUXM, DET>(p, tab_keys, tab_rows);
                 __syncthreads();
                 table_clear_keys<AUXM, DET>(tab_keys);   // the barrier at the top of the next round publishes it
