@@ -85,8 +85,10 @@ typedef struct DstParams {
     /* optional forward statistics: counters[0] += entries evaluated, counters[1] += hits composited */
     unsigned long long *counters;
     /* optional hit record (no counterpart in the reference): when non-NULL the forward trace stores every
-     * chunk's 16-entry hit buffer in it, and a backward trace given the same record replays the buffers
-     * instead of walking the BVH again (same results, no traversal).  Device memory, 8-byte aligned, sized
+     * chunk's 16-entry hit buffer in it, together with the colour it evaluated for every composited hit, and a
+     * backward trace given the same record replays the buffers instead of walking the BVH again and takes the
+     * colours instead of evaluating the spherical harmonics again (same results up to rounding of the gradient
+     * algebra, no traversal, no SH gather).  Device memory, 8-byte aligned, sized
      * with dst_hit_record_layout(); the caller zero-fills the first header_words words before the forward
      * call.  Word 0 then holds the number of blocks the forward trace asked for.  If that exceeds
      * hit_record_blocks the record is incomplete: the backward trace sees this ON THE DEVICE and walks the BVH
