@@ -284,6 +284,50 @@ def test_raw_launcher_calls_without_a_record(oracle, tracer):
     assert bwd[4].abs().max() == 0 and bwd[11].shape == (3000, 9) and bwd[11].abs().max() == 0
 
 
+def test_raw_launcher_calls_with_an_overflowed_and_with_a_damaged_record(oracle, tracer):
+    """Through the launchers directly, with records made by hand.  A record too small for the forward trace is seen
+    on the device: backward walks the BVH again and gives the oracle's gradients (not zeros).  A complete record whose
+    directory was wiped afterwards cannot be replayed: the call still returns, and word 1 of the record counts the
+    broken chains, which is how a caller can tell."""
+    import diff_surfel_tracing._C as binding
+    sc = S.scene_cube(P=3000, seed=6)
+    o, d = S.rays_cube(32, 40)
+    dev = "cuda"
+    g = {k: v.to(dev) for k, v in sc.items()}
+    ctx = tracer.optix_context
+    binding.build_acceleration_structure(ctx, g["vertices"], g["faces"], True)
+    e, eye, z3 = torch.empty(0, device=dev), torch.eye(4, device=dev), torch.zeros(3, device=dev)
+    common = (g["vertices"], z3, g["means3D"], g["shs"], 3, e, e, g["opacities"], g["scales"], 1.0, g["rotations"], e,
+              eye, eye, z3, False, False, 0, 0.0)
+    ug = upstream(32, 40, 2)
+    ups = [ug[k].to(dev) for k in ("rgb", "dpt", "acc", "norm")] + [torch.zeros(32, 40, 1, device=dev), ug["aux"].to(dev)]
+    s = oracle_scene(oracle, sc, o, d)
+    ref = oracle.forward(s, oracle.HITS_BVH_LEXI)
+    refg = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI)
+    refg64 = oracle.backward(s, ref, {k: v.numpy() for k, v in ug.items()}, oracle.HITS_BVH_LEXI, noise=True)
+    names = ("ray_o", "ray_d", "means3D", "grads3D", None, "shs", "colors_precomp", None, "opacities", "scales",
+             "rotations", None)
+
+    small = binding.HitRecord(32, 40, 1, 0.3, dev)          # room for a third of a block per wave
+    fwd = binding.trace_surfels(ctx, True, True, o.to(dev), d.to(dev), *common, hit_record=small)
+    bwd = binding.trace_surfels_backward(ctx, True, o.to(dev), d.to(dev), *common, *fwd[:7], *ups, hit_record=small)
+    torch.cuda.synchronize()
+    assert not small.complete() and small.broken_chains() == 0
+    np.testing.assert_array_equal(fwd[0].cpu().numpy(), ref["rgb"])
+    got = {k: t.cpu().numpy() for t, k in zip(bwd, names) if k is not None}
+    assert_gradients(got, {k: refg[k] for k in got}, refg64, GRAD_REL)
+
+    full = binding.HitRecord(32, 40, 1, 12.0, dev)
+    fwd = binding.trace_surfels(ctx, True, True, o.to(dev), d.to(dev), *common, hit_record=full)
+    torch.cuda.synchronize()
+    assert full.complete()
+    header = binding.HitRecord.layout(32, 40, 1, 12.0)[1]
+    full.words[2:header].zero_()                             # the directory: every chain now starts nowhere
+    binding.trace_surfels_backward(ctx, True, o.to(dev), d.to(dev), *common, *fwd[:7], *ups, hit_record=full)
+    torch.cuda.synchronize()
+    assert full.broken_chains() > 0
+
+
 def test_distortion_output_is_opt_in_and_equals_the_oracle(oracle, tracer):
     """`dist` is zero as in the reference unless SurfelTracer.distortion is set; then it is the 2DGS depth distortion
     of the primary ray, bit-equal to the oracle's, and nothing else changes."""
