@@ -1133,7 +1133,7 @@ __device__ __forceinline__ float *rec_store(const RecView &rv, int bounce, uint3
     if (blk >= rv.capacity) return nullptr;   // too small: the host sees the count and the backward pass re-traces
     uint64_t *b = rv.blocks + (size_t)blk * kRecBlockWords;
 #pragma unroll
-    for (int k = 0; k < kChunk; ++k) b[k * DST_WAVE + lane] = buf.e[k];
+    for (int k = 0; k < kChunk; ++k) __builtin_nontemporal_store(buf.e[k], b + k * DST_WAVE + lane);
     uint32_t *cnts = reinterpret_cast<uint32_t *>(b + kChunk * DST_WAVE);
     cnts[lane] = cnt;
     if (lane == 0) {
@@ -1251,7 +1251,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         // Replay runs one step ahead of itself: the entry of step it+1 is fetched while step it evaluates, and its
         // surfel's geometry while step it does its gradient algebra, so a step starts with its operands in registers
         // instead of two dependent trips to memory.
-        struct Ahead { uint64_t e; float m[3], s[2], q[4], o; } nx = {0ull, {0.f, 0.f, 0.f}, {1.f, 1.f}, {1.f, 0.f, 0.f, 0.f}, 0.f};
+        struct Ahead { uint64_t e; float m[3], s[2], q[4], o, c[3]; } nx = {0ull, {0.f, 0.f, 0.f}, {1.f, 1.f}, {1.f, 0.f, 0.f, 0.f}, 0.f, {0.f, 0.f, 0.f}};
         auto fetch_geometry = [&](bool want) {
             if (!want) return;
             const size_t gn = (size_t)(kb_idx(nx.e) >> 1);
@@ -1263,7 +1263,11 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         };
         if (REC && BWD) {
             const bool want = live && cnt > 0u;
-            if (want) nx.e = rec_block[lane_];
+            if (want) {
+                nx.e = __builtin_nontemporal_load(rec_block + lane_);
+                const float *cs = reinterpret_cast<const float *>(rec_block + kRecColourWord) + lane_;
+                for (int ch = 0; ch < 3; ++ch) nx.c[ch] = __builtin_nontemporal_load(cs + ch * DST_WAVE);
+            }
             fetch_geometry(want);
         }
 #pragma unroll 1
@@ -1277,7 +1281,12 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             const bool want_next = (REC && BWD) && live && it + 1 < kChunk && (uint32_t)(it + 1) < cnt;
             if (REC && BWD) {
                 e = cur.e;
-                if (want_next) nx.e = rec_block[(it + 1) * DST_WAVE + lane_];
+                if (want_next) {
+                    nx.e = __builtin_nontemporal_load(rec_block + (it + 1) * DST_WAVE + lane_);
+                    // (the colour slot of an entry that was not composited holds whatever was there: never used)
+                    const float *cs = reinterpret_cast<const float *>(rec_block + kRecColourWord) + (it + 1) * 3 * DST_WAVE + lane_;
+                    for (int ch = 0; ch < 3; ++ch) nx.c[ch] = __builtin_nontemporal_load(cs + ch * DST_WAVE);
+                }
             } else {
                 e = buf.e[0];
 #pragma unroll
@@ -1340,10 +1349,9 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 last_g = g;
                 w = alpha * Tp;
                 if (REC && BWD) {   // as the forward trace evaluated it
-                    const float *cs = reinterpret_cast<const float *>(rec_block + kRecColourWord) + it * 3 * DST_WAVE + lane_;
 #pragma unroll
                     for (int ch = 0; ch < 3; ++ch) {
-                        col[ch] = cs[ch * DST_WAVE];
+                        col[ch] = cur.c[ch];
                         // -0: clamped (a colour evaluated from SH is never negative; given colours may be)
                         neg[ch] = p.colors_precomp == nullptr && (__float_as_uint(col[ch]) >> 31) != 0u;
                     }
@@ -1359,7 +1367,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 if (REC && !BWD && rec_colours != nullptr) {
                     float *cs = rec_colours + it * 3 * DST_WAVE + lane_;
 #pragma unroll
-                    for (int ch = 0; ch < 3; ++ch) cs[ch * DST_WAVE] = neg[ch] ? -0.0f : col[ch];
+                    for (int ch = 0; ch < 3; ++ch) __builtin_nontemporal_store(neg[ch] ? -0.0f : col[ch], cs + ch * DST_WAVE);
                 }
                 run.C[0] += w * col[0];
                 run.C[1] += w * col[1];
