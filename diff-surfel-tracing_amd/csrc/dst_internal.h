@@ -54,12 +54,11 @@ static_assert(sizeof(DstLeaf) == 80, "leaf records are 20 dwords");
 // cannot pass the exact test; the walk fetches the 80-byte record and runs the exact test only if some lane
 // survives.  c = centroid, n = unit normal, fu/fv = dual vectors of the averaged half edges (s = fu.(P-c),
 // r = fv.(P-c): the corners sit at about (+-1, +-1)), mfu = max(|fu|, |fv|), lim0 = largest |s| or |r| of a
-// corner, a little enlarged, tdev = how far the corners leave the mean plane, enlarged (0 for a planar quad).
-// A degenerate quad gets mfu = inf: every ray survives.
+// corner, a little enlarged, tdev = how far the corners leave the mean plane, enlarged (0 for a planar quad),
+// rad = radius of a sphere around c that holds the quad.  A degenerate quad gets mfu = rad = inf: every ray survives.
 struct alignas(64) DstLeafPre {
     float c[3], n[3], fu[3], fv[3];
-    float mfu, lim0, tdev;
-    uint32_t pad;
+    float mfu, lim0, tdev, rad;
 };
 static_assert(sizeof(DstLeafPre) == 64, "one 16-dword scalar fetch");
 

@@ -344,7 +344,7 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
     cross_f(nrm, h1, t2);
     const float d1 = h1[0] * t1[0] + h1[1] * t1[1] + h1[2] * t1[2];
     const float d2 = h2[0] * t2[0] + h2[1] * t2[1] + h2[2] * t2[2];
-    float mfu = 0.f, lim0 = 0.f, dev = 0.f;
+    float mfu = 0.f, lim0 = 0.f, dev = 0.f, rad2 = 0.f;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
         fu[a] = t1[a] / d1;
@@ -357,12 +357,14 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
         lim0 = fmaxf(lim0, fabsf(fu[0] * w[0] + fu[1] * w[1] + fu[2] * w[2]));
         lim0 = fmaxf(lim0, fabsf(fv[0] * w[0] + fv[1] * w[1] + fv[2] * w[2]));
         dev = fmaxf(dev, fabsf(nrm[0] * w[0] + nrm[1] * w[1] + nrm[2] * w[2]));
+        rad2 = fmaxf(rad2, w[0] * w[0] + w[1] * w[1] + w[2] * w[2]);
     }
+    const float rad = sqrtf(rad2) * 1.002f;   // every point of the quad is within this distance of the centroid
     // A ray that meets the quad at less than 0.05 rad-ish from its plane skips the stand-in (trace kernels), so a
     // corner that is `dev` off the mean plane moves a hit by at most 20 dev along the plane; margins of 2.
     float tdev = 40.0f * dev;
     lim0 = lim0 * 1.002f + tdev * mfu;
-    const bool ok = isfinite(mfu) && isfinite(lim0) && isfinite(tdev) && isfinite(cen[0] + cen[1] + cen[2]) &&
+    const bool ok = isfinite(mfu) && isfinite(lim0) && isfinite(tdev) && isfinite(rad) && isfinite(cen[0] + cen[1] + cen[2]) &&
                     isfinite(nrm[0] + nrm[1] + nrm[2]) && nl > 0.f;
     float pr[16];
 #pragma unroll
@@ -375,7 +377,7 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
     pr[12] = ok ? mfu : INFINITY;
     pr[13] = ok ? lim0 : INFINITY;
     pr[14] = ok ? tdev : INFINITY;
-    pr[15] = 0.f;
+    pr[15] = ok ? rad : INFINITY;
     float4 *pdst = reinterpret_cast<float4 *>(&pre[i]);
 #pragma unroll
     for (int k = 0; k < 4; ++k) pdst[k] = make_float4(pr[4 * k], pr[4 * k + 1], pr[4 * k + 2], pr[4 * k + 3]);

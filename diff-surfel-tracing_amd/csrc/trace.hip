@@ -149,6 +149,7 @@ __device__ int dst_writelane(int value, int lane, int old) __asm("llvm.amdgcn.wr
 
 // ---- wave-uniform fetches ---------------------------------------------------------------------------------
 typedef const __attribute__((address_space(4))) uint32_t *const_u32_ptr;
+typedef __attribute__((address_space(3))) uint32_t *lds_u32;
 template <int N>
 __device__ __forceinline__ void load_uniform(const void *p, uint32_t (&out)[N]) {
     const_u32_ptr c = (const_u32_ptr)(uintptr_t)p;
@@ -208,6 +209,20 @@ __device__ __forceinline__ uint64_t slab_hit_fast(const RaySlabFast &s, float nx
     return __builtin_amdgcn_fcmpf(tn, tf, 5);   // 5 = ordered <=
 }
 
+// The same test as two masks: `far` = lanes whose ray meets the box at all (at a distance >= 0), result = those of
+// them that meet it within tmax.  Lanes that are switched off carry slab constants that fail both (see packet_walk).
+__device__ __forceinline__ uint64_t slab_hit_near_far(const RaySlabFast &s, float nx, float ny, float nz, float fx,
+                                                      float fy, float fz, float tmax, uint64_t &far) {
+    const float a = __builtin_fmaf(nx, s.ix, s.cnx), b = __builtin_fmaf(ny, s.iy, s.cny),
+                c = __builtin_fmaf(nz, s.iz, s.cnz);
+    const float e = __builtin_fmaf(fx, s.ix, s.cfx), f = __builtin_fmaf(fy, s.iy, s.cfy),
+                g = __builtin_fmaf(fz, s.iz, s.cfz);
+    const float tn = __builtin_fmaxf(__builtin_fmaxf(a, b), __builtin_fmaxf(c, 0.0f));
+    const float tf = __builtin_fminf(__builtin_fminf(e, f), g);
+    far = __builtin_amdgcn_fcmpf(tn, tf, 5);   // 5 = ordered <=
+    return far & __builtin_amdgcn_fcmpf(tn, tmax, 5);
+}
+
 // The 16 nearest hits of a lane, ascending.  One entry = (bits of t) << 32 | idx: t is positive, so the
 // unsigned 64-bit order is the (t, idx) lexicographic order and the content does not depend on the order in
 // which the BVH delivers candidates (ties in t resolve to ascending primitive index).
@@ -225,16 +240,18 @@ __device__ __forceinline__ void kbuf_reset(KBuf &b) {
 
 // Sorted insert in place: slot k keeps its entry if that is smaller than the new one, else takes the new one
 // (if the slot above kept its entry) or the entry from the slot above.
-__device__ __forceinline__ void kbuf_insert(KBuf &b, uint64_t x, bool on) {
+__device__ __forceinline__ void kbuf_insert(KBuf &b, uint64_t x_in, bool on) {
+    // a lane that inserts nothing offers the largest key: every slot keeps its entry (no per-slot gating)
+    const uint64_t x = on ? x_in : ~0ull;
     bool keep_k = b.e[kChunk - 1] < x;
 #pragma unroll
     for (int k = kChunk - 1; k >= 1; --k) {
         const bool keep_up = b.e[k - 1] < x;
         const uint64_t in = keep_up ? x : b.e[k - 1];
-        b.e[k] = (on && !keep_k) ? in : b.e[k];
+        b.e[k] = keep_k ? b.e[k] : in;
         keep_k = keep_up;
     }
-    b.e[0] = (on && !keep_k) ? x : b.e[0];
+    b.e[0] = keep_k ? b.e[0] : x;
 }
 
 #ifdef DST_STATS
@@ -269,7 +286,12 @@ __device__ __forceinline__ RayPre make_pre(F3 o, F3 d, float max_abs) {
 
 // The stand-in test of one quad for all lanes (about 28 instructions), as a lane mask: bit clear = that lane's ray
 // cannot pass the exact test (lanes that are switched off come back set or clear; the caller masks them).
-__device__ __forceinline__ uint64_t quad_may_hit(const uint32_t (&Q)[16], const RayPre &rp, F3 o, F3 d, float tmax) {
+// FAR: also `far`, the same without the limit tmax (lanes whose ray may hit the quad at any distance ahead); for a
+// grazing ray, whose distance to the plane says nothing, the quad counts as ahead unless the sphere around it lies
+// behind the origin.
+template <bool FAR>
+__device__ __forceinline__ uint64_t quad_may_hit(const uint32_t (&Q)[16], const RayPre &rp, F3 o, F3 d, float tmax,
+                                                 uint64_t live, uint64_t &far) {
 #define QF(k) __uint_as_float(Q[k])
     const float hx = QF(0) - o.x, hy = QF(1) - o.y, hz = QF(2) - o.z;
     const float qd = __builtin_fmaf(QF(5), d.z, __builtin_fmaf(QF(4), d.y, QF(3) * d.x));
@@ -282,10 +304,19 @@ __device__ __forceinline__ uint64_t quad_may_hit(const uint32_t (&Q)[16], const 
     const float lim = __builtin_fmaf(rp.padw, QF(12), QF(13));
     const float tpq = __builtin_fmaf(QF(14), rp.inv_dl, rp.tp);
     // every comparison is written so that a NaN keeps the ray in; the lane masks are combined without branches
-    const uint64_t flat = wave_ballot(__builtin_fabsf(qd) < rp.graze);
-    const uint64_t out = wave_ballot(m > lim) | wave_ballot(t < -tpq) | wave_ballot(__builtin_fmaf(t, 0.9999f, -tpq) > tmax);
+    uint64_t flat = wave_ballot(__builtin_fabsf(qd) < rp.graze);
+    const uint64_t out_base = wave_ballot(m > lim) | wave_ballot(t < -tpq);
+    const uint64_t out_t = wave_ballot(__builtin_fmaf(t, 0.9999f, -tpq) > tmax);
+    if (FAR) {
+        if ((flat & live) != 0ull) {
+            // (centre - o).d < -(radius + slack) |d|: every point of the quad is behind the origin
+            const float hd = __builtin_fmaf(hz, d.z, __builtin_fmaf(hy, d.y, hx * d.x));
+            flat &= ~wave_ballot(hd < -(QF(15) + rp.padw) * (20.0f * rp.graze));
+        }
+        far = flat | ~out_base;
+    }
 #undef QF
-    return flat | ~out;
+    return flat | ~(out_base | out_t);
 }
 
 // The exact test of one quad record for all lanes; hits are admitted into the lanes' buffers.
@@ -311,14 +342,17 @@ __device__ __forceinline__ void quad_exact(const uint32_t (&L)[19], F3 o, F3 d, 
 
 // A leaf group (up to DST_GROUP quads, consecutive records) against all lanes' rays.  The stand-in records of
 // two quads are fetched together, then the exact records of those that some lane's ray may hit, again together:
-// one trip to memory per stage instead of one per quad.
-__device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t first, uint32_t count, const RayPre &rp,
+// one trip to memory per stage instead of one per quad.  FAR: returns whether some live lane's ray may hit a quad
+// of the group at any distance ahead (the group has to be looked at again when the ray's next chunk is traced).
+template <bool FAR>
+__device__ __forceinline__ bool test_group(const DstAccelView &acc, uint32_t first, uint32_t count, const RayPre &rp,
                                            F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
 #ifdef DST_STATS
                                            , WaveStats &ws
 #endif
 ) {
     uint32_t q0 = 0;   // count >= 1
+    bool again = false;
 #pragma unroll 1
     do {
         const bool two = q0 + 1u < count;
@@ -329,8 +363,10 @@ __device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t fir
         STAT(ws.leaves += two ? 2 : 1;)
         const float tmax = kb_t(buf.e[kChunk - 1]);
         const uint64_t live = wave_ballot(active);
-        const uint64_t k0 = quad_may_hit(Q0, rp, o, d, tmax) & live;
-        const uint64_t k1 = two ? (quad_may_hit(Q1, rp, o, d, tmax) & live) : 0ull;
+        uint64_t f0 = 0ull, f1 = 0ull;
+        const uint64_t k0 = quad_may_hit<FAR>(Q0, rp, o, d, tmax, live, f0) & live;
+        const uint64_t k1 = two ? (quad_may_hit<FAR>(Q1, rp, o, d, tmax, live, f1) & live) : 0ull;
+        if (FAR) again = again || (((f0 | (two ? f1 : 0ull)) & live) != 0ull);
         uint32_t todo = (k0 != 0ull ? 1u : 0u) | (k1 != 0ull ? 2u : 0u);
 #pragma unroll 1
         while (todo != 0u) {
@@ -342,15 +378,34 @@ __device__ __forceinline__ void test_group(const DstAccelView &acc, uint32_t fir
         }
         q0 += 2;
     } while (DST_GROUP > 2 && q0 < count);   // groups of at most two quads: one pass, no loop
+    return again;
 }
+
+// Work list of a walk that can be resumed.  The rays of a wave are traced in chunks of 16 hits, each chunk from an
+// origin moved up to the last hit of the one before.  Instead of walking down from the root again, a walk writes
+// down what the next chunk can still need - the nodes it left with children that lie ahead of some ray but beyond
+// its 16th hit so far (with the children concerned), and the leaf groups it tested that hold a quad ahead of some
+// ray - and the next walk starts from that list.  What is ahead of a ray from the moved origin was ahead of it
+// before, and both tests have margins far above the rounding of the moved origin, so the list is a superset of
+// what a walk from the root would reach; the buffer's content does not depend on the order or on extra candidates.
+// An item is a leaf-group reference, or a node index with the children NOT to look at in bits 27..30.
+constexpr uint32_t kListCap = 512;            // items per list (a multiple of the wave size); a longer list is dropped
+constexpr uint32_t kListFresh = 0xFFFFFFFFu;  // n_in: no list, walk from the root
+constexpr uint32_t kListIndexBits = 27;       // node indices must fit below the excluded-children bits
+struct WalkList {
+    lds_u32 in, out;   // kListCap words each (LDS of this wave)
+    uint32_t n_in;     // items in `in`, or kListFresh
+    bool record;       // write `out` (false: plain walks from the root)
+};
 
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
 // to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow: nodes and quads
 // are fetched once per wave, the stack is two VGPRs addressed by lane (128 entries: the binary hierarchy
 // is at most 62 levels deep, a 4-wide step goes down two of them and defers at most three children: 96).
 // All active lanes share the direction signs `sgn` (bit a set = axis a negative), see slab_hit_fast.
+template <bool RESUME>
 __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySlab &slab, uint32_t sgn, F3 o, F3 d,
-                                            bool active, int rep, KBuf &buf, uint32_t &cnt
+                                            bool active, int rep, KBuf &buf, uint32_t &cnt, WalkList &wl
 #ifdef DST_STATS
                                             , WaveStats &ws
 #endif
@@ -363,26 +418,52 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
     fs.ix = slab.ix; fs.iy = slab.iy; fs.iz = slab.iz;
     fs.cnx = slab.nx - slab.wx; fs.cny = slab.ny - slab.wy; fs.cnz = slab.nz - slab.wz;
     fs.cfx = slab.nx + slab.wx; fs.cfy = slab.ny + slab.wy; fs.cfz = slab.nz + slab.wz;
+    const bool recording = RESUME && wl.record;
+    if (RESUME && !active) {   // a lane that is switched off meets no box: exit distance -inf on every axis
+        fs.ix = fs.iy = fs.iz = 0.f;
+        fs.cfx = fs.cfy = fs.cfz = -INFINITY;
+    }
     if (sgn & 1u) { onx = 48; ofx = 0; }
     if (sgn & 2u) { ony = 64; ofy = 16; }
     if (sgn & 4u) { onz = 80; ofz = 32; }
     uint32_t stack0 = 0u, stack1 = 0u;
     int sp = 0;
-    uint32_t ref = acc.root;
     // A well-formed hierarchy is walked in at most one step per node and per leaf group; the cap makes the
     // loops finite whatever the memory holds.  Two loops: the inner one goes down through nodes and never touches
     // the hit buffer, the outer one tests a leaf group and pops (with one loop around both, the compiler kept two
     // copies of the buffer's 32 registers and moved them back and forth at every leaf group).
     constexpr uint32_t kEnd = 0xFFFFFFFFu;   // not a reference: leaf bit set, impossible position
     uint32_t budget = 2u * acc.n_leaves + 8u;
+    // The work lists are read and written a page of 64 items at a time: lane k of a page register holds item k.
+    uint32_t in_page = 0u, out_page = 0u, in_pos = 0u, n_out = 0u;
+    const uint32_t n_in = (RESUME && wl.n_in != kListFresh) ? wl.n_in : 0u;
+    auto next_input = [&]() -> uint32_t {
+        if (!RESUME || in_pos >= n_in) return kEnd;
+        if ((in_pos & 63u) == 0u) in_page = wl.in[in_pos + lane];
+        const uint32_t v = __builtin_amdgcn_readlane(in_page, in_pos & 63u);
+        ++in_pos;
+        return v;
+    };
+    auto record = [&](uint32_t v) {
+        if (n_out < kListCap) {
+            out_page = (uint32_t)dst_writelane((int)v, n_out & 63u, (int)out_page);
+            if ((n_out & 63u) == 63u) wl.out[(n_out & ~63u) + lane] = out_page;
+        }
+        n_out = min(n_out + 1u, kListCap + 1u);
+    };
     auto pop = [&]() -> uint32_t {
-        if (sp == 0) return kEnd;
+        if (sp == 0) return next_input();
         --sp;
         const uint32_t a = __builtin_amdgcn_readlane(stack0, sp & 63), b = __builtin_amdgcn_readlane(stack1, sp & 63);
         return sp < 64 ? a : b;
     };
+    // node items of a list carry the children to leave out; plain references (stack, root) leave out none
+    const bool packed = RESUME && acc.n_leaves <= (1u << kListIndexBits);
+    uint32_t ref = (RESUME && wl.n_in != kListFresh) ? next_input() : acc.root;
     for (;;) {
         while ((ref & DST_LEAF_BIT) == 0u) {
+            const uint32_t excl = packed ? (ref >> kListIndexBits) : 0u;
+            if (packed) ref &= (1u << kListIndexBits) - 1u;
             if (budget == 0u || ref + 1u >= acc.n_leaves) {   // spent, or not a node of this hierarchy
                 ref = kEnd;
                 break;
@@ -394,6 +475,7 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
             uint32_t tail[5];
             load_uniform<5>(node + 96, tail);      // ref[4], count
             uint32_t hit = 0u;                     // bit k: some lane enters child k
+            uint32_t ahead = 0u;                   // bit k: child k lies ahead of some lane's ray, at any distance
             {
                 uint32_t NX[4], NY[4], NZ[4], FX[4], FY[4], FZ[4];
                 load_uniform<4>(node + onx, NX); load_uniform<4>(node + ony, NY); load_uniform<4>(node + onz, NZ);
@@ -403,13 +485,28 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                 asm volatile("" ::"s"(tail[0]), "s"(tail[1]), "s"(tail[2]), "s"(tail[3]), "s"(tail[4]), "s"(NX[0]));
 #pragma unroll
                 for (int k = 0; k < DST_WIDE; ++k) {
-                    float tn;
-                    const uint64_t h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
-                                                     __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
-                                                     __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn);
-                    hit |= (h != 0ull) ? (1u << k) : 0u;
+                    if (RESUME) {
+                        uint64_t far;
+                        const uint64_t h = slab_hit_near_far(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
+                                                             __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
+                                                             __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, far);
+                        hit |= (h != 0ull) ? (1u << k) : 0u;
+                        ahead |= (far != 0ull) ? (1u << k) : 0u;
+                    } else {
+                        float tn;
+                        const uint64_t h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
+                                                         __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
+                                                         __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn);
+                        hit |= (h != 0ull) ? (1u << k) : 0u;
+                    }
                 }
-                hit &= (1u << tail[4]) - 1u;       // unused slots are never entered
+                const uint32_t valid = ((1u << tail[4]) - 1u) & ~excl;   // unused slots are never entered
+                hit &= valid;
+                ahead &= valid;
+            }
+            if (recording) {
+                const uint32_t later = ahead & ~hit;   // beyond every ray's 16th hit so far: the next chunk's business
+                if (later != 0u) record(ref | ((~later & 15u) << kListIndexBits));
             }
             if (hit != 0u) {
                 // Children are taken in stored order: the first one that is hit next, the others deferred (last
@@ -434,8 +531,22 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
         --budget;
         const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
         if (first + count > acc.n_leaves) break;   // not a leaf group of this hierarchy
-        test_group(acc, first, count, rp, o, d, active, buf, cnt WSP);
+        const bool again = test_group<RESUME>(acc, first, count, rp, o, d, active, buf, cnt WSP);
+        if (recording && again) record(ref);
         ref = pop();
+    }
+    if (RESUME) {
+        if (recording) {
+            // a walk that stopped early (budget, damaged structure) or a list that overflowed leaves no list
+            const bool whole = n_out <= kListCap && budget != 0u && ref == kEnd;
+            if (whole && (n_out & 63u) != 0u) wl.out[(n_out & ~63u) + lane] = out_page;
+            wl.n_in = whole ? n_out : kListFresh;
+            const lds_u32 t = wl.in;
+            wl.in = wl.out;
+            wl.out = t;
+        } else {
+            wl.n_in = kListFresh;
+        }
     }
 }
 
@@ -459,7 +570,6 @@ constexpr uint32_t kWalkDone = 0xFFFFFFFFu;   // not a reference: leaf bit set w
 // The walk is a real function, so the compiler cannot see where its pointers lead: say it (global memory, LDS).
 typedef const __attribute__((address_space(1))) float *global_f32;
 typedef const __attribute__((address_space(1))) uint32_t *global_u32;
-typedef __attribute__((address_space(3))) uint32_t *lds_u32;
 #define LD3(p, k) f3((p)[(k)], (p)[(k) + 1], (p)[(k) + 2])
 // `shelf`: optional LDS for the first kLaneShelf stack entries of every lane ([entry][lane], conflict-free);
 // deeper entries, or all of them without a shelf, live in private memory.
@@ -573,9 +683,9 @@ __device__ __forceinline__ bool rays_run_together(F3 o, F3 d, bool active, float
     return wave_ballot(apart) == 0ull;
 }
 
-template <bool MIXED, bool SHELF>
+template <bool MIXED, bool SHELF, bool RESUME>
 __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
-                                           uint32_t &cnt, bool as_packet
+                                           uint32_t &cnt, bool as_packet, WalkList &wl
 #ifdef DST_STATS
                                            , WaveStats &ws
 #endif
@@ -600,12 +710,18 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
     // walked once per sign class present, each time with the lanes of that class only.
     const uint32_t my_sgn = (slab.ix < 0.f ? 1u : 0u) | (slab.iy < 0.f ? 2u : 0u) | (slab.iz < 0.f ? 4u : 0u);
     uint64_t todo = live;
+    if (RESUME) {
+        // a work list serves one walk per chunk: waves with several sign classes walk from the root every time
+        const uint32_t sgn0 = __builtin_amdgcn_readlane(my_sgn, __builtin_ctzll(live));
+        wl.record = wave_ballot(active && my_sgn != sgn0) == 0ull && acc.n_leaves <= (1u << kListIndexBits);
+        if (!wl.record) wl.n_in = kListFresh;
+    }
     while (todo != 0ull) {
         const int rep = __builtin_ctzll(todo);   // also the lane whose entry distances order the children
         const uint32_t sgn = __builtin_amdgcn_readlane(my_sgn, rep);
         const bool mine = active && my_sgn == sgn;
         todo &= ~wave_ballot(mine);
-        packet_walk(acc, slab, sgn, o, d, mine, rep, buf, cnt WSP);
+        packet_walk<RESUME>(acc, slab, sgn, o, d, mine, rep, buf, cnt, wl WSP);
     }
 }
 
@@ -1215,6 +1331,18 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     STAT(last_sh.t_alg = 0; last_sh.t_sh = 0;)
     // kernels built without the per-lane walk (MIXED false) take every wave as a packet
     const bool as_packet = (!MIXED || (REC && BWD)) ? true : rays_run_together(ro, rd, lane_on, max_abs);
+    // Forward: the walks of a bounce's later chunks resume from the list the walk before left (the backward
+    // re-trace has its LDS taken by the gradient table and walks from the root).
+#ifndef DST_RESUME
+#define DST_RESUME 1
+#endif
+    constexpr bool RESUME = !BWD && DST_RESUME;
+    __shared__ uint32_t s_list[RESUME ? kFwdWavesPerBlock * 2 * kListCap : 1];
+    WalkList wl;
+    wl.in = (lds_u32)(s_list + (RESUME ? (threadIdx.x / DST_WAVE) * 2 * kListCap : 0));
+    wl.out = wl.in + (RESUME ? kListCap : 0);
+    wl.n_in = kListFresh;
+    wl.record = false;
     uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
     for (;;) {
         // Backward: the four waves of the block take their chunks in step, so that between two rounds nobody
@@ -1242,7 +1370,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         } else {
             kbuf_reset(buf);
-            packet_knn<MIXED, MIXED && !BWD>(acc, max_abs, ot, rd, live, buf, cnt, as_packet WSP);
+            packet_knn<MIXED, MIXED && !BWD, RESUME>(acc, max_abs, ot, rd, live, buf, cnt, as_packet, wl WSP);
             if (REC && !BWD) rec_colours = rec_store(rv, bounce, rec_pos, buf, cnt);
         }
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
