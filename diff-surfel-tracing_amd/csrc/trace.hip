@@ -685,7 +685,7 @@ __device__ __forceinline__ bool rays_run_together(F3 o, F3 d, bool active, float
 
 template <bool MIXED, bool SHELF, bool RESUME>
 __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
-                                           uint32_t &cnt, bool as_packet, WalkList &wl
+                                           uint32_t &cnt, bool as_packet, WalkList &wl, uint32_t *shelf
 #ifdef DST_STATS
                                            , WaveStats &ws
 #endif
@@ -697,10 +697,8 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
         KBuf mine = buf;   // a copy the call may keep in memory; the caller's buffer stays in registers
         uint32_t n = cnt;
         // forward kernels (one wave per workgroup, no other LDS) give the walk an LDS shelf for its stacks
-        __shared__ uint32_t s_shelf[SHELF ? kFwdWavesPerBlock * kLaneShelf * DST_WAVE : 1];
         const LaneWalkAccel view = {acc.leaves, acc.wide, acc.n_leaves, acc.root};
-        lane_walk(view, slab, o, d, active, mine, n,
-                  SHELF ? s_shelf + (threadIdx.x / DST_WAVE) * (kLaneShelf * DST_WAVE) : nullptr);
+        lane_walk(view, slab, o, d, active, mine, n, SHELF ? shelf : nullptr);
         buf = mine;
         cnt = n;
         return;
@@ -1337,9 +1335,15 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
 #define DST_RESUME 1
 #endif
     constexpr bool RESUME = !BWD && DST_RESUME;
-    __shared__ uint32_t s_list[RESUME ? kFwdWavesPerBlock * 2 * kListCap : 1];
+    // One LDS area per wave serves the packet walk's two lists or the per-lane walk's stack shelf: all chunks of
+    // a bounce use the same walk, and a bounce starts without a list.
+    constexpr bool SHELF = MIXED && !BWD;
+    constexpr uint32_t kWaveLds = (SHELF && (uint32_t)(kLaneShelf * DST_WAVE) > 2u * kListCap) ? (uint32_t)(kLaneShelf * DST_WAVE)
+                                                                                               : (RESUME ? 2u * kListCap : 1u);
+    __shared__ uint32_t s_list[(RESUME || SHELF) ? kFwdWavesPerBlock * kWaveLds : 1];
+    uint32_t *const wave_lds = s_list + ((RESUME || SHELF) ? (threadIdx.x / DST_WAVE) * kWaveLds : 0);
     WalkList wl;
-    wl.in = (lds_u32)(s_list + (RESUME ? (threadIdx.x / DST_WAVE) * 2 * kListCap : 0));
+    wl.in = (lds_u32)wave_lds;
     wl.out = wl.in + (RESUME ? kListCap : 0);
     wl.n_in = kListFresh;
     wl.record = false;
@@ -1370,7 +1374,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         } else {
             kbuf_reset(buf);
-            packet_knn<MIXED, MIXED && !BWD, RESUME>(acc, max_abs, ot, rd, live, buf, cnt, as_packet, wl WSP);
+            packet_knn<MIXED, SHELF, RESUME>(acc, max_abs, ot, rd, live, buf, cnt, as_packet, wl, wave_lds WSP);
             if (REC && !BWD) rec_colours = rec_store(rv, bounce, rec_pos, buf, cnt);
         }
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
