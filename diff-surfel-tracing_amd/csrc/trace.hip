@@ -157,6 +157,55 @@ __device__ __forceinline__ void load_uniform(const void *p, uint32_t (&out)[N]) 
     for (int k = 0; k < N; ++k) out[k] = c[k];
 }
 
+// A whole traversal node in one trip: the six face arrays picked by byte offset (scalar-register offsets, so no
+// address arithmetic per array), the child references and the child count, and one wait for all of them.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void load_node(const void *node, uint32_t onx, uint32_t ony, uint32_t onz, uint32_t ofx,
+                                          uint32_t ofy, uint32_t ofz, u32x4 &NX, u32x4 &NY, u32x4 &NZ, u32x4 &FX,
+                                          u32x4 &FY, u32x4 &FZ, u32x4 &refs, uint32_t &count) {
+    asm volatile(
+        "s_load_dwordx4 %0, %8, %9\n\t"
+        "s_load_dwordx4 %1, %8, %10\n\t"
+        "s_load_dwordx4 %2, %8, %11\n\t"
+        "s_load_dwordx4 %3, %8, %12\n\t"
+        "s_load_dwordx4 %4, %8, %13\n\t"
+        "s_load_dwordx4 %5, %8, %14\n\t"
+        "s_load_dwordx4 %6, %8, 0x60\n\t"
+        "s_load_dword %7, %8, 0x70\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&s"(NX), "=&s"(NY), "=&s"(NZ), "=&s"(FX), "=&s"(FY), "=&s"(FZ), "=&s"(refs), "=&s"(count)
+        : "s"(node), "s"(onx), "s"(ony), "s"(onz), "s"(ofx), "s"(ofy), "s"(ofz)
+        : "memory");
+}
+// Two consecutive 64-byte records (the stand-ins of a leaf group's two quads), or one 80-byte quad record, in one
+// trip: left to itself the compiler splits these fetches and waits for the first part before asking for the rest.
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ void load_record_pair(const void *p, u32x16 &a, u32x16 &b) {
+    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(a), "=&s"(b)
+                 : "s"(p)
+                 : "memory");
+}
+__device__ __forceinline__ void load_quad_record(const void *p, u32x16 &a, u32x4 &b) {
+    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx4 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(a), "=&s"(b)
+                 : "s"(p)
+                 : "memory");
+}
+// bits = 2 * bits + (mask != 0): one compare and one add-with-carry per lane mask.
+__device__ __forceinline__ uint32_t shift_in_any(uint32_t bits, uint64_t mask) {
+    asm("s_cmp_lg_u64 %1, 0\n\ts_addc_u32 %0, %0, %0" : "+s"(bits) : "s"(mask) : "scc");
+    return bits;
+}
+// The same for two masks at once: hit takes (a & b) != 0, ahead takes b != 0 (the and sets the carry itself).
+__device__ __forceinline__ void shift_in_near_far(uint32_t &hit, uint32_t &ahead, uint64_t a, uint64_t b) {
+    uint64_t both;
+    asm("s_and_b64 %2, %3, %4\n\ts_addc_u32 %0, %0, %0\n\ts_cmp_lg_u64 %4, 0\n\ts_addc_u32 %1, %1, %1"
+        : "+s"(hit), "+s"(ahead), "=&s"(both)
+        : "s"(a), "s"(b)
+        : "scc");
+}
+
 struct RaySlab {   // per-lane precomputation for the conservative slab test
     float ix, iy, iz;     // 1/d, with tiny components pushed away from zero
     float nx, ny, nz;     // -o * (1/d)
@@ -290,7 +339,7 @@ __device__ __forceinline__ RayPre make_pre(F3 o, F3 d, float max_abs) {
 // grazing ray, whose distance to the plane says nothing, the quad counts as ahead unless the sphere around it lies
 // behind the origin.
 template <bool FAR>
-__device__ __forceinline__ uint64_t quad_may_hit(const uint32_t (&Q)[16], const RayPre &rp, F3 o, F3 d, float tmax,
+__device__ __forceinline__ uint64_t quad_may_hit(const u32x16 &Q, const RayPre &rp, F3 o, F3 d, float tmax,
                                                  uint64_t live, uint64_t &far) {
 #define QF(k) __uint_as_float(Q[k])
     const float hx = QF(0) - o.x, hy = QF(1) - o.y, hz = QF(2) - o.z;
@@ -320,18 +369,20 @@ __device__ __forceinline__ uint64_t quad_may_hit(const uint32_t (&Q)[16], const 
 }
 
 // The exact test of one quad record for all lanes; hits are admitted into the lanes' buffers.
-__device__ __forceinline__ void quad_exact(const uint32_t (&L)[19], F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
+__device__ __forceinline__ void quad_exact(const u32x16 &La, const u32x4 &Lb, F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
 #ifdef DST_STATS
                                            , WaveStats &ws
 #endif
 ) {
     STAT(ws.t_plan++;)
-#define LF3(k) f3(__uint_as_float(L[k]), __uint_as_float(L[(k) + 1]), __uint_as_float(L[(k) + 2]))
+#define LW(k) ((k) < 16 ? La[(k) & 15] : Lb[((k) - 16) & 3])
+#define LF3(k) f3(__uint_as_float(LW(k)), __uint_as_float(LW((k) + 1)), __uint_as_float(LW((k) + 2)))
     float t = 0.f;
     uint32_t tri = 0u;
     const bool hit = active && ray_quad(o, d, LF3(0), LF3(3), LF3(6), LF3(9), LF3(12), LF3(15), t, tri);
 #undef LF3
-    const uint64_t x = kb_pack(t, 2u * L[18] + tri);
+    const uint64_t x = kb_pack(t, 2u * LW(18) + tri);
+#undef LW
     const bool adm = hit && (x < buf.e[kChunk - 1]);
     if (wave_ballot(adm) != 0ull) {
         STAT(ws.leaf_any++;)
@@ -357,9 +408,8 @@ __device__ __forceinline__ bool test_group(const DstAccelView &acc, uint32_t fir
     do {
         const bool two = q0 + 1u < count;
         // the record after the last quad of the structure exists (the array has one spare record)
-        uint32_t Q0[16], Q1[16];
-        load_uniform<16>(&acc.pre[first + q0], Q0);
-        load_uniform<16>(&acc.pre[first + q0 + 1u], Q1);
+        u32x16 Q0, Q1;
+        load_record_pair(&acc.pre[first + q0], Q0, Q1);
         STAT(ws.leaves += two ? 2 : 1;)
         const float tmax = kb_t(buf.e[kChunk - 1]);
         const uint64_t live = wave_ballot(active);
@@ -372,9 +422,10 @@ __device__ __forceinline__ bool test_group(const DstAccelView &acc, uint32_t fir
         while (todo != 0u) {
             const uint32_t k = (todo & 1u) ? 0u : 1u;
             todo &= ~(1u << k);
-            uint32_t L[19];
-            load_uniform<19>(&acc.leaves[first + q0 + k], L);
-            quad_exact(L, o, d, active, buf, cnt WSP);
+            u32x16 La;
+            u32x4 Lb;
+            load_quad_record(&acc.leaves[first + q0 + k], La, Lb);
+            quad_exact(La, Lb, o, d, active, buf, cnt WSP);
         }
         q0 += 2;
     } while (DST_GROUP > 2 && q0 < count);   // groups of at most two quads: one pass, no loop
@@ -473,31 +524,28 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
             STAT(ws.nodes++;)
             const float tmax = active ? kb_t(buf.e[kChunk - 1]) : -1.0f;
             uint32_t tail[5];
-            load_uniform<5>(node + 96, tail);      // ref[4], count
             uint32_t hit = 0u;                     // bit k: some lane enters child k
             uint32_t ahead = 0u;                   // bit k: child k lies ahead of some lane's ray, at any distance
             {
-                uint32_t NX[4], NY[4], NZ[4], FX[4], FY[4], FZ[4];
-                load_uniform<4>(node + onx, NX); load_uniform<4>(node + ony, NY); load_uniform<4>(node + onz, NZ);
-                load_uniform<4>(node + ofx, FX); load_uniform<4>(node + ofy, FY); load_uniform<4>(node + ofz, FZ);
-                // one trip to memory per node: without this the compiler fetches the references and the count only
-                // when they are used, two more waits behind the first
-                asm volatile("" ::"s"(tail[0]), "s"(tail[1]), "s"(tail[2]), "s"(tail[3]), "s"(tail[4]), "s"(NX[0]));
+                u32x4 NX, NY, NZ, FX, FY, FZ, refs;
+                load_node(node, onx, ony, onz, ofx, ofy, ofz, NX, NY, NZ, FX, FY, FZ, refs, tail[4]);
+                tail[0] = refs[0]; tail[1] = refs[1]; tail[2] = refs[2]; tail[3] = refs[3];
 #pragma unroll
-                for (int k = 0; k < DST_WIDE; ++k) {
+                for (int k = DST_WIDE - 1; k >= 0; --k) {   // last child first: its bit is shifted up the furthest
+                    const float a = __builtin_fmaf(__uint_as_float(NX[k]), fs.ix, fs.cnx),
+                                b = __builtin_fmaf(__uint_as_float(NY[k]), fs.iy, fs.cny),
+                                c = __builtin_fmaf(__uint_as_float(NZ[k]), fs.iz, fs.cnz);
+                    const float e = __builtin_fmaf(__uint_as_float(FX[k]), fs.ix, fs.cfx),
+                                f = __builtin_fmaf(__uint_as_float(FY[k]), fs.iy, fs.cfy),
+                                g = __builtin_fmaf(__uint_as_float(FZ[k]), fs.iz, fs.cfz);
+                    const float tn = __builtin_fmaxf(__builtin_fmaxf(a, b), __builtin_fmaxf(c, 0.0f));
                     if (RESUME) {
-                        uint64_t far;
-                        const uint64_t h = slab_hit_near_far(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
-                                                             __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
-                                                             __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, far);
-                        hit |= (h != 0ull) ? (1u << k) : 0u;
-                        ahead |= (far != 0ull) ? (1u << k) : 0u;
+                        // met at all (at a distance >= 0) / met within tmax; lanes that are switched off fail both
+                        const float tf = __builtin_fminf(__builtin_fminf(e, f), g);
+                        shift_in_near_far(hit, ahead, __builtin_amdgcn_fcmpf(tn, tmax, 5), __builtin_amdgcn_fcmpf(tn, tf, 5));
                     } else {
-                        float tn;
-                        const uint64_t h = slab_hit_fast(fs, __uint_as_float(NX[k]), __uint_as_float(NY[k]),
-                                                         __uint_as_float(NZ[k]), __uint_as_float(FX[k]),
-                                                         __uint_as_float(FY[k]), __uint_as_float(FZ[k]), tmax, tn);
-                        hit |= (h != 0ull) ? (1u << k) : 0u;
+                        const float tf = __builtin_fminf(__builtin_fminf(e, f), __builtin_fminf(g, tmax));
+                        hit = shift_in_any(hit, __builtin_amdgcn_fcmpf(tn, tf, 5));   // 5 = ordered <=
                     }
                 }
                 const uint32_t valid = ((1u << tail[4]) - 1u) & ~excl;   // unused slots are never entered
@@ -512,16 +560,28 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
                 // Children are taken in stored order: the first one that is hit next, the others deferred (last
                 // first).  Ordering them by entry distance was measured: 3 % fewer visits, but the scalar work of
                 // the sort costs more than those visits.
+                const uint32_t rest = hit & (hit - 1u);   // the hit children after the first one (never child 0)
+                if (__builtin_expect(sp + 3 <= DST_WAVE, 1)) {
+                    // Without branches: each candidate is written at the top of the stack and the top moves up only
+                    // if the child was hit (an entry above the top is dead, so a write there does no harm).
+                    stack0 = (uint32_t)dst_writelane((int)tail[3], sp, (int)stack0);
+                    sp += (int)((rest >> 3) & 1u);
+                    stack0 = (uint32_t)dst_writelane((int)tail[2], sp, (int)stack0);
+                    sp += (int)((rest >> 2) & 1u);
+                    stack0 = (uint32_t)dst_writelane((int)tail[1], sp, (int)stack0);
+                    sp += (int)((rest >> 1) & 1u);
+                } else {
 #define DST_PUSH(v)                                                                                          \
     {                                                                                                        \
         if (sp < 64) stack0 = (uint32_t)dst_writelane((int)(v), sp, (int)stack0);               \
         else stack1 = (uint32_t)dst_writelane((int)(v), sp - 64, (int)stack1);                  \
         sp = min(sp + 1, 2 * DST_WAVE - 1);                                                                  \
     }
-                if ((hit & 8u) && (hit & 7u)) DST_PUSH(tail[3])
-                if ((hit & 4u) && (hit & 3u)) DST_PUSH(tail[2])
-                if ((hit & 2u) && (hit & 1u)) DST_PUSH(tail[1])
+                    if (rest & 8u) DST_PUSH(tail[3])
+                    if (rest & 4u) DST_PUSH(tail[2])
+                    if (rest & 2u) DST_PUSH(tail[1])
 #undef DST_PUSH
+                }
                 ref = (hit & 1u) ? tail[0] : ((hit & 2u) ? tail[1] : ((hit & 4u) ? tail[2] : tail[3]));
             } else {
                 ref = pop();
@@ -1331,15 +1391,13 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     const bool as_packet = (!MIXED || (REC && BWD)) ? true : rays_run_together(ro, rd, lane_on, max_abs);
     // Forward: the walks of a bounce's later chunks resume from the list the walk before left (the backward
     // re-trace has its LDS taken by the gradient table and walks from the root).
-#ifndef DST_RESUME
-#define DST_RESUME 1
-#endif
-    constexpr bool RESUME = !BWD && DST_RESUME;
+    constexpr bool RESUME = !BWD;
     // One LDS area per wave serves the packet walk's two lists or the per-lane walk's stack shelf: all chunks of
     // a bounce use the same walk, and a bounce starts without a list.
     constexpr bool SHELF = MIXED && !BWD;
-    constexpr uint32_t kWaveLds = (SHELF && (uint32_t)(kLaneShelf * DST_WAVE) > 2u * kListCap) ? (uint32_t)(kLaneShelf * DST_WAVE)
-                                                                                               : (RESUME ? 2u * kListCap : 1u);
+    constexpr uint32_t kListWords = 2u * kListCap;
+    constexpr uint32_t kWaveLds = (SHELF && (uint32_t)(kLaneShelf * DST_WAVE) > kListWords) ? (uint32_t)(kLaneShelf * DST_WAVE)
+                                                                                            : (RESUME ? kListWords : 1u);
     __shared__ uint32_t s_list[(RESUME || SHELF) ? kFwdWavesPerBlock * kWaveLds : 1];
     uint32_t *const wave_lds = s_list + ((RESUME || SHELF) ? (threadIdx.x / DST_WAVE) * kWaveLds : 0);
     WalkList wl;
