@@ -147,6 +147,51 @@ def test_coplanar_ties_and_dense_stacks(oracle, tracer):
                      noise=ref["grads_noise"]["rotations"][:, live_cols])
 
 
+def _with_scales(sc, factor):
+    """The scene with every surfel `factor` times larger (quads rebuilt)."""
+    out = dict(sc)
+    out["scales"] = sc["scales"] * factor
+    out["vertices"], out["faces"] = S.get_triangles(sc["means3D"], out["scales"], sc["rotations"])
+    return out
+
+
+def test_later_chunks_where_a_work_list_cannot_help(oracle, tracer):
+    """The forward walk of a ray's second and later chunks starts from the list the walk before left (nodes and leaf
+    groups still ahead of some ray).  Cases that leave that path: more leaf groups ahead of one wave than a list holds
+    (the walk falls back to the root), rays that graze their quads (no usable plane distance: a quad stays on the list
+    until the sphere around it is behind the origin), and waves whose rays differ in direction signs (no list at all).
+    Outputs must be the oracle's bits in each."""
+    from test_oracle_scalar import _tie_scene
+    # (a) 2400 coplanar quads, 1200 leaf groups, nearly all of them ahead of every ray of the wave at once
+    sc = _tie_scene(2400, seed=5)
+    o = torch.stack(torch.meshgrid(torch.linspace(-0.2, 0.2, 16), torch.linspace(-0.2, 0.2, 16), indexing="ij"), -1)
+    o = torch.cat([o, torch.full((16, 16, 1), 3.0)], -1).contiguous()
+    d = torch.tensor([0.0, 0.0, -1.0]).expand(16, 16, 3).contiguous()
+    ref, _ = check_case(oracle, tracer, sc, o, d, grads=False)
+    assert ref["n_proc"].max() > 16
+    # (b) sixty large parallel quads 4 mm apart, met at 1.1 to 2.6 degrees: dozens of hits per ray, all of them grazing
+    P = 60
+    gen = torch.Generator().manual_seed(11)
+    means = torch.cat([0.2 * torch.rand(P, 2, generator=gen), (0.4 - 0.004 * torch.arange(1, P + 1)).reshape(P, 1)], -1)
+    scales = torch.ones(P, 2)
+    rot = torch.tensor([1.0, 0.0, 0.0, 0.0]).repeat(P, 1)
+    v, f = S.get_triangles(means, scales, rot)
+    sc = {"means3D": means, "scales": scales, "rotations": rot, "opacities": torch.full((P, 1), 0.1),
+          "colors_precomp": torch.rand(P, 3, generator=gen), "vertices": v, "faces": f}
+    ys, slopes = torch.meshgrid(torch.linspace(-1.0, 1.0, 16), torch.linspace(0.02, 0.045, 16), indexing="ij")
+    o = torch.stack([torch.full_like(ys, -2.5), ys, torch.full_like(ys, 0.4)], -1).contiguous()
+    d = torch.stack([torch.ones_like(ys), torch.zeros_like(ys), -slopes], -1).contiguous()
+    ref, _ = check_case(oracle, tracer, sc, o, d, grads=False)
+    assert ref["n_proc"].max() > 32
+    # (c) the image centre of a pinhole camera: the four tiles around it hold rays of four sign classes; surfels
+    # enlarged until those rays need several chunks
+    sc = _with_scales(S.scene_cube(P=6000, seed=7, colors=True), 4.0)
+    o, d = S.rays_cube(32, 32)
+    ref, _ = check_case(oracle, tracer, sc, o, d, grads=False)
+    centre = ref["n_proc"].reshape(32, 32)[8:24, 8:24]
+    assert centre.max() > 32
+
+
 def test_refit_equals_rebuild(oracle, tracer):
     sc = S.scene_lidar(P=30000, seed=2, aux=4)
     o, d = S.rays_lidar(beams=16, azimuths=128)
