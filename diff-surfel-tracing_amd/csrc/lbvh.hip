@@ -137,12 +137,16 @@ __global__ void k_morton(const float4 *__restrict__ centroids, const DstBounds *
     float4 c = centroids[g];
     const float cc[3] = {c.x, c.y, c.z};
     uint32_t q[3];
+    // Cubic cells: one scale for the three axes (the longest extent).  With a scale per axis a flat scene (a 200 m
+    // ground with 4 m of height) gets cells of 20 cm x 20 cm x 4 mm, and the hierarchy splits in height long before
+    // it has separated what lies far apart on the ground.
+    float ext = 0.f;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) ext = fmaxf(ext, ord2f(bounds->hi[a]) - ord2f(bounds->lo[a]));
+    const float s = (ext > 0.f && ext < INFINITY) ? 1024.0f / ext : 0.f;
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        float lo = ord2f(bounds->lo[a]), hi = ord2f(bounds->hi[a]);
-        float ext = hi - lo;
-        float s = (ext > 0.f && ext < INFINITY) ? 1024.0f / ext : 0.f;
-        float x = (cc[a] - lo) * s;
+        float x = (cc[a] - ord2f(bounds->lo[a])) * s;
         x = fminf(fmaxf(x, 0.f), 1023.f);  // NaN -> 0
         q[a] = (uint32_t)x;
     }
