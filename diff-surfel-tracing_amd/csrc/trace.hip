@@ -1038,9 +1038,15 @@ struct GradSink {
         const uint32_t lane = __lane_id();
         const float *a = stage + (lane & 15u) * kStageStride + (lane & 48u);
         v4f acc = {0.f, 0.f, 0.f, 0.f};
+        // all sixteen operands are asked for before the first product: left alone, the compiler reads two, waits,
+        // multiplies, reads the next two, ... - eight trips to LDS one after the other per tile
+        float av[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) av[m] = a[m];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int m = 0; m < 16; ++m)
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[m], ((members >> m) & 1u) ? 1.0f : 0.0f, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[m], ((members >> m) & 1u) ? 1.0f : 0.0f, acc, 0, 0, 0);
         // acc[r] = column 16*tile + 4*(lane/16) + r summed over the rays of group lane%16
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
