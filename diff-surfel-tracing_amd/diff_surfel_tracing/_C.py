@@ -225,7 +225,10 @@ class OptiXStateWrapper:
 
     def acquire_record(self, H, W, mtd_alloc, device):
         self.update_record_estimate()
-        words = HitRecord.layout(H, W, mtd_alloc, self.record_blocks_per_wave)[0]
+        # every bounce of a path opens at least one block per wave: before anything has been learned from a finished
+        # forward trace, a multi-bounce record is sized for that many more
+        per_wave = max(self.record_blocks_per_wave, 4.0 * (mtd_alloc + 1))
+        words = HitRecord.layout(H, W, mtd_alloc, per_wave)[0]
         if 8 * words > self.record_max_bytes:
             return None
         device = torch.device(device)
@@ -243,7 +246,7 @@ class OptiXStateWrapper:
                 storage = torch.empty(words + words // 8, dtype=torch.int64, device=device)
             except torch.OutOfMemoryError:
                 return None
-        return HitRecord(H, W, mtd_alloc, self.record_blocks_per_wave, device, storage=storage)
+        return HitRecord(H, W, mtd_alloc, per_wave, device, storage=storage)
 
     def release_record(self, rec):
         if rec is None or rec.words is None:
