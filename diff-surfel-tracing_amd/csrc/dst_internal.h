@@ -97,6 +97,9 @@ struct dst_ctx {
     uint32_t *flags = nullptr;                                // arrival counters of the bottom-up fit
     int32_t *quad_ids = nullptr;                              // 4 vertex ids per surfel (int4)
     float *centroids = nullptr;                               // 4 floats per surfel
+    // boxes of leaf ranges for the fit by look-up: per leaf its own box, the union of its 64-leaf block up to it and
+    // from it on (6 floats each), and the unions of 2^l consecutive blocks for every l
+    float *range_lbox = nullptr, *range_pbox = nullptr, *range_sbox = nullptr, *range_table = nullptr;
     uint32_t *keys[2] = {nullptr, nullptr}, *vals[2] = {nullptr, nullptr};
     uint32_t *tile_hist = nullptr;
     size_t tile_hist_elems = 0;

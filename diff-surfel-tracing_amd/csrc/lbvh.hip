@@ -173,23 +173,20 @@ __global__ void k_radix_hist(const uint32_t *__restrict__ keys, uint32_t *__rest
         for (int d = lane; d < kRadix; d += DST_WAVE) tile_hist[(size_t)d * n_tiles + tile] = hist[w][d];
 }
 
-// Exclusive scan of `len` counters in place, one block.
-__global__ void k_scan_exclusive(uint32_t *data, uint32_t len) {
-    // one block walks the array in coalesced slabs of blockDim.x * 4 entries and carries the running total
+// Exclusive scan of the tile counters in two steps: block d scans the row of digit d (one counter per tile) in place
+// and leaves the row's total in row_total[d]; a second, tiny kernel turns the 256 totals into the digits' start
+// positions, which the scatter adds to a tile's entry.  (One block walking all 256 x tiles counters took 0.14 ms per
+// pass at a million keys: a fifth of the whole build.)
+__global__ void k_scan_rows(uint32_t *tile_hist, uint32_t *row_total, uint32_t n_tiles) {
     __shared__ uint32_t wave_sum[1024 / DST_WAVE];
     __shared__ uint32_t carry_s;
-    constexpr uint32_t kPer = 4u;
-    const uint32_t t = threadIdx.x, nt = blockDim.x, lane = t % DST_WAVE, w = t / DST_WAVE, nw = nt / DST_WAVE;
+    uint32_t *data = tile_hist + (size_t)blockIdx.x * n_tiles;
+    const uint32_t t = threadIdx.x, nt = blockDim.x, lane = t % DST_WAVE, w = t / DST_WAVE;
     if (t == 0) carry_s = 0u;
     __syncthreads();
-    for (uint32_t base = 0; base < len; base += nt * kPer) {
-        const uint32_t i = base + t * kPer;
-        uint32_t v[kPer];
-#pragma unroll
-        for (int k = 0; k < (int)kPer; ++k) v[k] = (i + k < len) ? data[i + k] : 0u;
-        uint32_t mine = 0u;
-#pragma unroll
-        for (int k = 0; k < (int)kPer; ++k) mine += v[k];
+    for (uint32_t base = 0; base < n_tiles; base += nt) {
+        const uint32_t i = base + t;
+        const uint32_t mine = i < n_tiles ? data[i] : 0u;
         uint32_t incl = mine;   // inclusive scan over the wave
 #pragma unroll
         for (int off = 1; off < DST_WAVE; off <<= 1) {
@@ -200,26 +197,36 @@ __global__ void k_scan_exclusive(uint32_t *data, uint32_t len) {
         __syncthreads();
         uint32_t before = carry_s;
         for (uint32_t k = 0; k < w; ++k) before += wave_sum[k];
-        uint32_t run = before + incl - mine;
-#pragma unroll
-        for (int k = 0; k < (int)kPer; ++k) {
-            if (i + k < len) data[i + k] = run;
-            run += v[k];
-        }
+        if (i < n_tiles) data[i] = before + incl - mine;
         __syncthreads();
-        if (t == nt - 1) carry_s = run;   // the last thread's running total is the slab's
+        if (t == nt - 1) carry_s = before + incl;   // the last thread's running total is the slab's
         __syncthreads();
     }
+    if (t == 0) row_total[blockIdx.x] = carry_s;
+}
+__global__ void k_scan_digits(uint32_t *row_total) {   // one block of kRadix threads, in place, exclusive
+    __shared__ uint32_t s[kRadix];
+    const uint32_t t = threadIdx.x;
+    s[t] = row_total[t];
+    __syncthreads();
+    for (uint32_t off = 1; off < kRadix; off <<= 1) {
+        const uint32_t add = t >= off ? s[t - off] : 0u;
+        __syncthreads();
+        s[t] += add;
+        __syncthreads();
+    }
+    row_total[t] = s[t] - row_total[t];
 }
 
 __global__ void k_radix_scatter(const uint32_t *__restrict__ keys_in, const uint32_t *__restrict__ vals_in,
                                 uint32_t *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
-                                const uint32_t *__restrict__ tile_hist, uint32_t n, uint32_t n_tiles, int shift) {
+                                const uint32_t *__restrict__ tile_hist, const uint32_t *__restrict__ digit_start,
+                                uint32_t n, uint32_t n_tiles, int shift) {
     __shared__ uint32_t base[kBlock / DST_WAVE][kRadix];
     const int w = threadIdx.x / DST_WAVE, lane = threadIdx.x % DST_WAVE;
     const uint32_t tile = blockIdx.x * (kBlock / DST_WAVE) + w;
     if (tile < n_tiles)
-        for (int d = lane; d < kRadix; d += DST_WAVE) base[w][d] = tile_hist[(size_t)d * n_tiles + tile];
+        for (int d = lane; d < kRadix; d += DST_WAVE) base[w][d] = tile_hist[(size_t)d * n_tiles + tile] + digit_start[d];
     __syncthreads();
     if (tile >= n_tiles) return;
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -387,24 +394,128 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
     for (int k = 0; k < 4; ++k) pdst[k] = make_float4(pr[4 * k], pr[4 * k + 1], pr[4 * k + 2], pr[4 * k + 3]);
 }
 
+// ---- boxes of leaf ranges without climbing the tree ---------------------------------------------------------
+// A node of the hierarchy covers a contiguous range of leaves, so its children's boxes are range unions of leaf
+// boxes, and those can be looked up instead of being carried up the tree by threads that wait for each other:
+// leaves are cut into blocks of 64 (one wave of the kernels that write the leaf records); every leaf stores the
+// union of its block up to itself (`pbox`) and from itself on (`sbox`), a table holds the unions of 2^l consecutive
+// blocks for every l, and a range is: rest of its first block + start of its last block + two table entries for
+// the blocks between - or, inside one block, a loop over at most 62 leaf boxes.  min/max are exact, so the boxes
+// are the same bits as those of the climbing fit.
+constexpr int kRangeBlock = DST_WAVE;
+struct RangeBoxes {
+    float *lbox, *pbox, *sbox;   // 6 floats per leaf: lo[3], hi[3]
+    float *table;                // [level][block][6]
+};
+__device__ __forceinline__ void box_join(float (&a)[6], const float *b) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        a[k] = fminf(a[k], b[k]);
+        a[3 + k] = fmaxf(a[3 + k], b[3 + k]);
+    }
+}
+__device__ __forceinline__ void box_store(float *dst, const float (&b)[6]) {
+    float2 *d = reinterpret_cast<float2 *>(dst);
+    d[0] = make_float2(b[0], b[1]);
+    d[1] = make_float2(b[2], b[3]);
+    d[2] = make_float2(b[4], b[5]);
+}
+// Called by ALL 64 lanes of a wave whose lane l holds leaf position base + l (`valid`: that position exists).
+__device__ __forceinline__ void wave_range_boxes(const float (&c)[4][3], bool valid, uint32_t i, uint32_t n,
+                                                 const RangeBoxes &rb) {
+    const uint32_t lane = threadIdx.x % DST_WAVE;
+    float box[6], pre[6], suf[6];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        box[a] = valid ? fminf(fminf(c[0][a], c[1][a]), fminf(c[2][a], c[3][a])) : INFINITY;
+        box[3 + a] = valid ? fmaxf(fmaxf(c[0][a], c[1][a]), fmaxf(c[2][a], c[3][a])) : -INFINITY;
+    }
+#pragma unroll
+    for (int k = 0; k < 6; ++k) pre[k] = suf[k] = box[k];
+#pragma unroll
+    for (int off = 1; off < DST_WAVE; off <<= 1) {
+#pragma unroll
+        for (int k = 0; k < 6; ++k) {
+            const float up = __shfl_up(pre[k], off), down = __shfl_down(suf[k], off);
+            if ((int)lane >= off) pre[k] = k < 3 ? fminf(pre[k], up) : fmaxf(pre[k], up);
+            if ((int)lane + off < DST_WAVE) suf[k] = k < 3 ? fminf(suf[k], down) : fmaxf(suf[k], down);
+        }
+    }
+    if (!valid) return;
+    box_store(rb.lbox + 6 * (size_t)i, box);
+    box_store(rb.pbox + 6 * (size_t)i, pre);
+    box_store(rb.sbox + 6 * (size_t)i, suf);
+    if (lane == DST_WAVE - 1 || i == n - 1u) box_store(rb.table + 6 * (size_t)(i / kRangeBlock), pre);   // level 0: whole blocks
+}
+// table[level][b] = union of blocks b .. b + 2^level - 1 (entries that would run past the last block stay unused)
+__global__ void k_range_table_level(float *table, uint32_t n_blocks, int level) {
+    const uint32_t b = blockIdx.x * blockDim.x + threadIdx.x, half = 1u << (level - 1);
+    if (b + 2u * half > n_blocks) return;
+    const float *lo = table + ((size_t)(level - 1) * n_blocks + b) * 6, *hi = lo + 6 * (size_t)half;
+    float box[6];
+#pragma unroll
+    for (int k = 0; k < 6; ++k) box[k] = lo[k];
+    box_join(box, hi);
+    box_store(table + ((size_t)level * n_blocks + b) * 6, box);
+}
+__device__ __forceinline__ void range_box(const RangeBoxes &rb, uint32_t n_blocks, uint32_t a, uint32_t b, float (&box)[6]) {
+    const uint32_t ba = a / kRangeBlock, bb = b / kRangeBlock;
+    if (ba == bb) {
+        const float *src = rb.lbox + 6 * (size_t)a;
+#pragma unroll
+        for (int k = 0; k < 6; ++k) box[k] = src[k];
+        for (uint32_t j = a + 1u; j <= b; ++j) box_join(box, rb.lbox + 6 * (size_t)j);
+        return;
+    }
+    const float *s = rb.sbox + 6 * (size_t)a;
+#pragma unroll
+    for (int k = 0; k < 6; ++k) box[k] = s[k];
+    box_join(box, rb.pbox + 6 * (size_t)b);
+    if (bb > ba + 1u) {
+        const uint32_t x = ba + 1u, y = bb - 1u;
+        const int l = 31 - __clz(y - x + 1u);
+        box_join(box, rb.table + ((size_t)l * n_blocks + x) * 6);
+        box_join(box, rb.table + ((size_t)l * n_blocks + (y + 1u - (1u << l))) * 6);
+    }
+}
+// Fit by look-up: node i's children cover leaves first..split and split+1..last (split = the child reference itself,
+// see k_karras).
+__global__ void k_fit_ranges(DstNode *nodes, RangeBoxes rb, uint32_t n_blocks, uint32_t n_internal) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_internal) return;
+    DstNode &nd = nodes[i];
+    const uint32_t first = nd.first, last = nd.last, split = nd.c0 & ~DST_LEAF_BIT;
+    float b0[6], b1[6];
+    range_box(rb, n_blocks, first, split, b0);
+    range_box(rb, n_blocks, split + 1u, last, b1);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        nd.lo0[k] = b0[k]; nd.hi0[k] = b0[3 + k];
+        nd.lo1[k] = b1[k]; nd.hi1[k] = b1[3 + k];
+    }
+}
+
 // Leaf records in Morton order (also the whole of a refit's geometry update).
 __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
                             const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
-                            DstLeafPre *__restrict__ pre, uint32_t n) {
-    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    uint32_t g = sorted_ids[i];
-    int4 q = quad_ids[g];
-    const int ids[4] = {q.x, q.y, q.z, q.w};
-    float c[4][3];
+                            DstLeafPre *__restrict__ pre, RangeBoxes rb, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool valid = i < n;   // every lane stays for the wave-wide scans of the boxes
+    float c[4][3] = {};
+    if (valid) {
+        uint32_t g = sorted_ids[i];
+        int4 q = quad_ids[g];
+        const int ids[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const float *v = vertices + (size_t)ids[k] * 3;
-        c[k][0] = v[0];
-        c[k][1] = v[1];
-        c[k][2] = v[2];
+        for (int k = 0; k < 4; ++k) {
+            const float *v = vertices + (size_t)ids[k] * 3;
+            c[k][0] = v[0];
+            c[k][1] = v[1];
+            c[k][2] = v[2];
+        }
+        write_leaf(c, g, i, leaves, pre);
     }
-    write_leaf(c, g, i, leaves, pre);
+    if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
 }
 
 // The same for a refit straight from the surfel parameters: the four corners of surfel g are
@@ -417,9 +528,15 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
 __global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const float *__restrict__ scales,
                                          const float *__restrict__ rotations, const uint32_t *__restrict__ sorted_ids,
                                          DstLeaf *__restrict__ leaves, DstLeafPre *__restrict__ pre,
-                                         float *__restrict__ vertices_out, DstBounds *__restrict__ bounds, uint32_t n) {
+                                         float *__restrict__ vertices_out, DstBounds *__restrict__ bounds,
+                                         RangeBoxes rb, uint32_t n) {
     float mabs = 0.f;
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+    // wave-uniform trip count: every lane stays for the wave-wide scans of the boxes
+    for (uint32_t base = blockIdx.x * blockDim.x + (threadIdx.x & ~(DST_WAVE - 1u)); base < n; base += gridDim.x * blockDim.x) {
+        const uint32_t i = base + (threadIdx.x & (DST_WAVE - 1u));
+        const bool valid = i < n;
+        float c[4][3] = {};
+        if (valid) {
         const uint32_t g = sorted_ids[i];
         const float q0 = rotations[4 * (size_t)g], q1 = rotations[4 * (size_t)g + 1], q2 = rotations[4 * (size_t)g + 2],
                     q3 = rotations[4 * (size_t)g + 3];
@@ -430,7 +547,6 @@ __global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const 
         const float v[3] = {(2.f * (x * y - w * z)) * sy, (1.f - 2.f * (x * x + z * z)) * sy, (2.f * (y * z + w * x)) * sy};
         const float m[3] = {means[3 * (size_t)g], means[3 * (size_t)g + 1], means[3 * (size_t)g + 2]};
         const float sa[4] = {-3.f, -3.f, 3.f, 3.f}, sb[4] = {3.f, -3.f, 3.f, -3.f};
-        float c[4][3];
 #pragma unroll
         for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -445,6 +561,8 @@ __global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const 
             dst[2] = make_float4(c[2][2], c[3][0], c[3][1], c[3][2]);
         }
         write_leaf(c, g, i, leaves, pre);
+        }
+        if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
     }
     mabs = wave_max(mabs);
     if ((threadIdx.x & (DST_WAVE - 1)) == 0 && mabs > 0.f && mabs < INFINITY)
@@ -580,11 +698,20 @@ int ensure_capacity(dst_ctx *ctx, uint32_t P) {
     DST_HIP(ctx, hipMalloc((void **)&ctx->flags, sizeof(uint32_t) * n));
     DST_HIP(ctx, hipMalloc((void **)&ctx->quad_ids, sizeof(int32_t) * 4 * n));
     DST_HIP(ctx, hipMalloc((void **)&ctx->centroids, sizeof(float) * 4 * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->range_lbox, sizeof(float) * 6 * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->range_pbox, sizeof(float) * 6 * n));
+    DST_HIP(ctx, hipMalloc((void **)&ctx->range_sbox, sizeof(float) * 6 * n));
+    {
+        const size_t n_blocks = (n + kRangeBlock - 1) / kRangeBlock;
+        size_t levels = 1;
+        while ((size_t(2) << (levels - 1)) <= n_blocks) ++levels;
+        DST_HIP(ctx, hipMalloc((void **)&ctx->range_table, sizeof(float) * 6 * n_blocks * levels));
+    }
     for (int k = 0; k < 2; ++k) {
         DST_HIP(ctx, hipMalloc((void **)&ctx->keys[k], sizeof(uint32_t) * n));
         DST_HIP(ctx, hipMalloc((void **)&ctx->vals[k], sizeof(uint32_t) * n));
     }
-    ctx->tile_hist_elems = tiles * kRadix;
+    ctx->tile_hist_elems = tiles * kRadix + kRadix;
     DST_HIP(ctx, hipMalloc((void **)&ctx->tile_hist, sizeof(uint32_t) * ctx->tile_hist_elems));
     if (!ctx->bounds) DST_HIP(ctx, hipMalloc((void **)&ctx->bounds, sizeof(DstBounds)));
     if (!ctx->bounds_host) DST_HIP(ctx, hipHostMalloc((void **)&ctx->bounds_host, sizeof(DstBounds), hipHostMallocDefault));
@@ -617,20 +744,22 @@ uint32_t *dst_static_scratch(const dst_ctx *ctx) {
 }
 
 // Stable LSD radix sort of (key, value) pairs, 32-bit keys, four 8-bit passes; the sorted pairs end in buffer 0.
-// tile_hist holds 256 counters per 1024 keys.  Used by the BVH build (Morton codes) and by the ray ordering.
+// tile_hist holds 256 counters per 1024 keys and 256 more for the digits' start positions (dst_sort_hist_elems).  Used by the BVH build (Morton codes) and by the ray ordering.
 void dst_sort_pairs(uint32_t *keys[2], uint32_t *vals[2], uint32_t *tile_hist, uint32_t n, hipStream_t stream) {
     const uint32_t tiles = (n + kTile - 1) / kTile;
     const uint32_t tile_blocks = (tiles + (kBlock / DST_WAVE) - 1) / (kBlock / DST_WAVE);
     int src = 0;
     for (int shift = 0; shift < 32; shift += kRadixBits) {
         hipLaunchKernelGGL(k_radix_hist, dim3(tile_blocks), dim3(kBlock), 0, stream, keys[src], tile_hist, n, tiles, shift);
-        hipLaunchKernelGGL(k_scan_exclusive, dim3(1), dim3(1024), 0, stream, tile_hist, tiles * kRadix);
+        uint32_t *digit_start = tile_hist + (size_t)tiles * kRadix;   // kRadix words behind the tile counters
+        hipLaunchKernelGGL(k_scan_rows, dim3(kRadix), dim3(1024), 0, stream, tile_hist, digit_start, tiles);
+        hipLaunchKernelGGL(k_scan_digits, dim3(1), dim3(kRadix), 0, stream, digit_start);
         hipLaunchKernelGGL(k_radix_scatter, dim3(tile_blocks), dim3(kBlock), 0, stream, keys[src], vals[src],
-                           keys[1 - src], vals[1 - src], tile_hist, n, tiles, shift);
+                           keys[1 - src], vals[1 - src], tile_hist, digit_start, n, tiles, shift);
         src = 1 - src;
     }
 }
-size_t dst_sort_hist_elems(uint32_t n) { return (size_t)((n + kTile - 1) / kTile) * kRadix; }
+size_t dst_sort_hist_elems(uint32_t n) { return (size_t)((n + kTile - 1) / kTile) * kRadix + kRadix; }
 
 void dst_lbvh_free(dst_ctx *ctx) {
     auto rel = [](auto *&p) {
@@ -646,6 +775,10 @@ void dst_lbvh_free(dst_ctx *ctx) {
     rel(ctx->flags);
     rel(ctx->quad_ids);
     rel(ctx->centroids);
+    rel(ctx->range_lbox);
+    rel(ctx->range_pbox);
+    rel(ctx->range_sbox);
+    rel(ctx->range_table);
     rel(ctx->keys[0]);
     rel(ctx->keys[1]);
     rel(ctx->vals[0]);
@@ -670,6 +803,11 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
         if (rc) return rc;
         ctx->n_leaves = P;
     }
+    // The fit looks the boxes up (k_fit_ranges); a caller that brings its own arrival counters (the refit that
+    // allocates nothing) gets the climbing fit, which needs nothing else.
+    const bool by_ranges = fit_flags == nullptr;
+    RangeBoxes rb = {nullptr, nullptr, nullptr, nullptr};
+    if (by_ranges) rb = RangeBoxes{ctx->range_lbox, ctx->range_pbox, ctx->range_sbox, ctx->range_table};
     if (fit_flags == nullptr) fit_flags = ctx->flags;   // after ensure_capacity: a first build allocates them there
     if (fit_flags == nullptr || ctx->nodes == nullptr || ctx->leaves == nullptr || ctx->pre == nullptr ||
         ctx->vals[0] == nullptr)
@@ -683,7 +821,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     if (surfels != nullptr) {
         // refit from the surfel parameters: corners, leaf records and the coordinate bound in one kernel
         hipLaunchKernelGGL(k_leaf_fill_from_surfels, setup_grid, dim3(kBlock), 0, stream, surfels->means, surfels->scales,
-                           surfels->rotations, ctx->vals[0], ctx->leaves, ctx->pre, surfels->vertices_out, ctx->bounds, n);
+                           surfels->rotations, ctx->vals[0], ctx->leaves, ctx->pre, surfels->vertices_out, ctx->bounds, rb, n);
     } else if (rebuild)
         hipLaunchKernelGGL(k_quad_setup<true>, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
                            quad_ids, centroids, ctx->bounds, n);
@@ -705,10 +843,18 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     }
     if (surfels == nullptr)
         hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0],
-                           ctx->leaves, ctx->pre, n);
-    hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, fit_flags, 0u, n);
-    hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
-                       fit_flags, ctx->leaves, n);
+                           ctx->leaves, ctx->pre, rb, n);
+    if (by_ranges) {
+        const uint32_t n_blocks = (n + kRangeBlock - 1) / kRangeBlock;
+        for (int level = 1; (2u << (level - 1)) <= n_blocks; ++level)
+            hipLaunchKernelGGL(k_range_table_level, grid_for(n_blocks), dim3(kBlock), 0, stream, ctx->range_table, n_blocks, level);
+        if (n > 1)
+            hipLaunchKernelGGL(k_fit_ranges, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, rb, n_blocks, n - 1);
+    } else {
+        hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, fit_flags, 0u, n);
+        hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
+                           fit_flags, ctx->leaves, n);
+    }
     if (n > DST_GROUP)
         hipLaunchKernelGGL(k_widen, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, ctx->wide, n - 1);
     DST_HIP(ctx, hipGetLastError());
