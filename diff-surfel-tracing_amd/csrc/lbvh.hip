@@ -52,45 +52,82 @@ __global__ void k_fill_u32(uint32_t *p, uint32_t v, uint32_t n) {
     if (i < n) p[i] = v;
 }
 
-// Per surfel: resolve the quad's four vertex ids through the triangle buffer (build) or reuse them
-// (refit), then reduce centroid bounds and the largest |coordinate|.
-template <bool REBUILD>
+// Largest |coordinate| of a block's quads -> bounds->max_abs: the waves meet in LDS, one atomic per block (atomics of
+// many waves to one word are served one by one).  Every thread of the block calls it.
+__device__ __forceinline__ void block_max_abs(float mabs, DstBounds *bounds) {
+    __shared__ float s_m[kBlock / DST_WAVE];
+    mabs = wave_max(mabs);
+    if ((threadIdx.x & (DST_WAVE - 1)) == 0) s_m[threadIdx.x / DST_WAVE] = mabs;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x / DST_WAVE); ++w) mabs = fmaxf(mabs, s_m[w]);
+        if (mabs > 0.f && mabs < INFINITY) atomicMax(&bounds->max_abs, __float_as_uint(mabs));
+    }
+}
+
+// The four corners of a quad: rows ids[0..3] of the vertex buffer; rows 4g..4g+3 in order (the usual layout) are
+// 48 consecutive bytes and come as three 16-byte loads.
+__device__ __forceinline__ void load_corners(const float *__restrict__ vertices, int4 q, uint32_t g, float (&c)[4][3]) {
+    if (q.x == (int)(4u * g) && q.y == q.x + 1 && q.z == q.x + 2 && q.w == q.x + 3 &&
+        (reinterpret_cast<uintptr_t>(vertices) & 15u) == 0u) {
+        const float4 *v = reinterpret_cast<const float4 *>(vertices + 12 * (size_t)g);
+        const float4 a = v[0], b = v[1], d = v[2];
+        c[0][0] = a.x; c[0][1] = a.y; c[0][2] = a.z; c[1][0] = a.w;
+        c[1][1] = b.x; c[1][2] = b.y; c[2][0] = b.z; c[2][1] = b.w;
+        c[2][2] = d.x; c[3][0] = d.y; c[3][1] = d.z; c[3][2] = d.w;
+        return;
+    }
+    const int ids[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float *v = vertices + (size_t)ids[k] * 3;
+        c[k][0] = v[0];
+        c[k][1] = v[1];
+        c[k][2] = v[2];
+    }
+}
+
+// Build only.  Per surfel: resolve the quad's four vertex ids through the triangle buffer, then reduce the centroid
+// bounds (Morton codes) and the largest |coordinate| (the trace kernels' padding).  A refit keeps the ids and gets
+// the coordinate bound from the kernel that writes the leaf records.
 __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vertices,
                              const int32_t *__restrict__ triangles, int4 *__restrict__ quad_ids,
                              float4 *__restrict__ centroids, DstBounds *__restrict__ bounds, uint32_t P) {
-    // grid-stride: a wave ends with seven atomics on the same seven words, and those are served one by one,
-    // so each wave takes many surfels
+    // grid-stride: a block ends with seven atomics on the same seven words, and those are served one by one,
+    // so each block takes many surfels
+    __shared__ float s_lo[kBlock / DST_WAVE][3], s_hi[kBlock / DST_WAVE][3];
     float cen[3] = {INFINITY, INFINITY, INFINITY}, cenh[3] = {-INFINITY, -INFINITY, -INFINITY};
     float mabs = 0.f;
     for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < P; g += gridDim.x * blockDim.x) {
         float lo[3] = {INFINITY, INFINITY, INFINITY}, hi[3] = {-INFINITY, -INFINITY, -INFINITY};
-        int4 q;
-        if (REBUILD) {
-            const int32_t *t = triangles + (size_t)g * 6;
-            q = make_int4(t[0], t[1], t[2], t[5]);
-            bool bad = (t[3] != t[1]) || (t[4] != t[2]);
-            bad |= (uint32_t)q.x >= n_vertices || (uint32_t)q.y >= n_vertices || (uint32_t)q.z >= n_vertices ||
-                   (uint32_t)q.w >= n_vertices;
-            if (bad) {
-                atomicOr(&bounds->bad_topology, 1u);
-                q = make_int4(0, 0, 0, 0);
-            } else if (q.x != (int)(4u * g) || q.y != q.x + 1 || q.z != q.x + 2 || q.w != q.x + 3) {
-                atomicOr(&bounds->bad_topology, 2u);   // valid, but not rows 4g..4g+3 in order
-            }
-            quad_ids[g] = q;
+        const int32_t *t = triangles + (size_t)g * 6;   // 24 bytes per surfel: three 8-byte loads where the buffer allows
+        int2 ta, tb, tc;
+        if ((reinterpret_cast<uintptr_t>(triangles) & 7u) == 0u) {
+            const int2 *t2 = reinterpret_cast<const int2 *>(t);
+            ta = t2[0]; tb = t2[1]; tc = t2[2];
         } else {
-            q = quad_ids[g];
+            ta = make_int2(t[0], t[1]); tb = make_int2(t[2], t[3]); tc = make_int2(t[4], t[5]);
         }
-        const int ids[4] = {q.x, q.y, q.z, q.w};
+        int4 q = make_int4(ta.x, ta.y, tb.x, tc.y);
+        bool bad = (tb.y != ta.y) || (tc.x != tb.x);
+        bad |= (uint32_t)q.x >= n_vertices || (uint32_t)q.y >= n_vertices || (uint32_t)q.z >= n_vertices ||
+               (uint32_t)q.w >= n_vertices;
+        if (bad) {
+            atomicOr(&bounds->bad_topology, 1u);
+            q = make_int4(0, 0, 0, 0);
+        } else if (q.x != (int)(4u * g) || q.y != q.x + 1 || q.z != q.x + 2 || q.w != q.x + 3) {
+            atomicOr(&bounds->bad_topology, 2u);   // valid, but not rows 4g..4g+3 in order
+        }
+        quad_ids[g] = q;
+        float c[4][3];
+        load_corners(vertices, q, g, c);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const float *v = vertices + (size_t)ids[k] * 3;
 #pragma unroll
             for (int a = 0; a < 3; ++a) {
-                float c = v[a];
-                lo[a] = fminf(lo[a], c);
-                hi[a] = fmaxf(hi[a], c);
-                mabs = fmaxf(mabs, fabsf(c));
+                lo[a] = fminf(lo[a], c[k][a]);
+                hi[a] = fmaxf(hi[a], c[k][a]);
+                mabs = fmaxf(mabs, fabsf(c[k][a]));
             }
         }
         float4 c4;
@@ -108,17 +145,28 @@ __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vert
         cen[a] = wave_min(cen[a]);
         cenh[a] = wave_max(cenh[a]);
     }
-    mabs = wave_max(mabs);
+    const int w = threadIdx.x / DST_WAVE;
     if ((threadIdx.x & (DST_WAVE - 1)) == 0) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-            if (cen[a] <= cenh[a]) {  // skips empty and NaN-only waves
-                atomicMin(&bounds->lo[a], f2ord(cen[a]));
-                atomicMax(&bounds->hi[a], f2ord(cenh[a]));
-            }
+            s_lo[w][a] = cen[a];
+            s_hi[w][a] = cenh[a];
         }
-        if (mabs > 0.f && mabs < INFINITY) atomicMax(&bounds->max_abs, __float_as_uint(mabs));
     }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const int a = threadIdx.x;
+        float l = INFINITY, h = -INFINITY;
+        for (int k = 0; k < (int)(blockDim.x / DST_WAVE); ++k) {
+            l = fminf(l, s_lo[k][a]);
+            h = fmaxf(h, s_hi[k][a]);
+        }
+        if (l <= h) {  // skips empty and NaN-only blocks
+            atomicMin(&bounds->lo[a], f2ord(l));
+            atomicMax(&bounds->hi[a], f2ord(h));
+        }
+    }
+    block_max_abs(mabs, bounds);
 }
 
 __device__ __forceinline__ uint32_t spread10(uint32_t v) {
@@ -498,24 +546,22 @@ __global__ void k_fit_ranges(DstNode *nodes, RangeBoxes rb, uint32_t n_blocks, u
 // Leaf records in Morton order (also the whole of a refit's geometry update).
 __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
                             const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
-                            DstLeafPre *__restrict__ pre, RangeBoxes rb, uint32_t n) {
+                            DstLeafPre *__restrict__ pre, RangeBoxes rb, DstBounds *__restrict__ bounds, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     const bool valid = i < n;   // every lane stays for the wave-wide scans of the boxes
     float c[4][3] = {};
+    float mabs = 0.f;
     if (valid) {
-        uint32_t g = sorted_ids[i];
-        int4 q = quad_ids[g];
-        const int ids[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float *v = vertices + (size_t)ids[k] * 3;
-            c[k][0] = v[0];
-            c[k][1] = v[1];
-            c[k][2] = v[2];
-        }
+        const uint32_t g = sorted_ids[i];
+        load_corners(vertices, quad_ids[g], g, c);
         write_leaf(c, g, i, leaves, pre);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int a = 0; a < 3; ++a) mabs = fmaxf(mabs, fabsf(c[k][a]));
     }
     if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
+    if (bounds != nullptr) block_max_abs(mabs, bounds);   // a refit: the coordinate bound of the moved quads
 }
 
 // The same for a refit straight from the surfel parameters: the four corners of surfel g are
@@ -823,10 +869,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
         hipLaunchKernelGGL(k_leaf_fill_from_surfels, setup_grid, dim3(kBlock), 0, stream, surfels->means, surfels->scales,
                            surfels->rotations, ctx->vals[0], ctx->leaves, ctx->pre, surfels->vertices_out, ctx->bounds, rb, n);
     } else if (rebuild)
-        hipLaunchKernelGGL(k_quad_setup<true>, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
-                           quad_ids, centroids, ctx->bounds, n);
-    else
-        hipLaunchKernelGGL(k_quad_setup<false>, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
+        hipLaunchKernelGGL(k_quad_setup, setup_grid, dim3(kBlock), 0, stream, vertices, n_vertices, triangles,
                            quad_ids, centroids, ctx->bounds, n);
 
     if (rebuild) {
@@ -843,7 +886,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     }
     if (surfels == nullptr)
         hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0],
-                           ctx->leaves, ctx->pre, rb, n);
+                           ctx->leaves, ctx->pre, rb, rebuild ? nullptr : ctx->bounds, n);
     if (by_ranges) {
         const uint32_t n_blocks = (n + kRangeBlock - 1) / kRangeBlock;
         for (int level = 1; (2u << (level - 1)) <= n_blocks; ++level)
