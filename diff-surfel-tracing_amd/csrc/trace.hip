@@ -27,6 +27,13 @@ constexpr int kWavesPerBlock = 4;
 #define DST_FWD_WPB 1
 #endif
 constexpr int kFwdWavesPerBlock = DST_FWD_WPB;   // 1 or kWavesPerBlock
+#ifndef DST_STRIP_FWD
+#define DST_STRIP_FWD 8   // width of the column strips the blocks of an image grid are walked in (0: row-major)
+#endif
+#ifndef DST_STRIP_BWD
+#define DST_STRIP_BWD 8
+#endif
+constexpr uint32_t kStripMinBlocks = 4096;   // forward: strips only for grids of at least this many blocks (see launch())
 
 __device__ const float SH0 = 0.28209479177387814f;
 __device__ const float SH1 = 0.4886025119029199f;
@@ -1671,7 +1678,7 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
 template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x,
-                                           const uint32_t *__restrict__ ray_order) {
+                                           const uint32_t *__restrict__ ray_order, uint32_t strip_width) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     constexpr int kTableRows = RowLayout<AUXM>::rows;
@@ -1701,12 +1708,25 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         bid = (blockIdx.x >> 5) * 8u + (blockIdx.x & 7u);
         wv = (blockIdx.x >> 3) & 3u;
     }
-    // Blocks keep the dispatch order (row-major over the 16x16 pixel tiles).  Two re-numberings that give each of the
-    // 8 XCDs (workgroup number mod 8, an L2 each) its own part of the image were measured on the 1080p room scene
-    // and are slower: a band or whole rows per XCD (+15 % / +8 % forward: eight distant image regions in flight,
-    // eight times more distinct BVH data in the shared last-level cache), and compact neighbouring patches of 2x4
-    // to 8x16 blocks per XCD inside super-tiles (+1 % to +13 %, more with larger patches).
-    const uint32_t bx = bid % btiles_x, by = bid / btiles_x;
+    // (Measured slower than the strips below, on the 1080p room scene: a band or whole rows of the image per XCD,
+    // +15 % / +8 % forward - eight distant image regions in flight, eight times more distinct BVH data in the shared
+    // last-level cache - and compact patches of 2x4 to 8x16 blocks per XCD inside super-tiles, +1 % to +13 %.)
+    // Image grids are walked in column strips eight blocks wide, row by row inside a strip.  Workgroups go to the
+    // eight XCDs in turn, so in a full strip XCD q works its way down column q: the tiles an XCD has in flight are
+    // vertical neighbours and meet the same BVH nodes in that XCD's own L2 (row-major order over a 120-block-wide image
+    // gave an XCD blocks eight columns apart: forward 8.5 -> 8.1 ms on the 1080p room scene).  The last strip may be
+    // narrower; its blocks are spread over all XCDs like the others.  The launcher chooses the width (launch()).
+    const uint32_t kStrip = strip_width;   // 0: row-major
+    uint32_t bx = bid % btiles_x, by = bid / btiles_x;
+    if (kStrip != 0u && th_log2 != 0) {
+        const uint32_t rows = (tiles_y + 1u) / 2u, per_strip = kStrip * rows;
+        const uint32_t strip = bid / per_strip, r = bid % per_strip;
+        if (strip * kStrip < btiles_x) {   // (blocks past the grid keep the row-major numbers and leave below)
+            const uint32_t w = min(kStrip, btiles_x - strip * kStrip);
+            bx = strip * kStrip + r % w;
+            by = r / w;
+        }
+    }
     const bool flat = th_log2 == 0;   // a ray list: tiles of 1x64 rays, a block = four consecutive tiles
     if (flat ? by >= 1u : 2u * by >= tiles_y) return;   // padding of the forward grid (whole blocks)
     RecView rv = {nullptr, nullptr, nullptr, 0u};
@@ -1935,14 +1955,14 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
 template <int AUXM, bool REC, bool MIXED, bool EXTRAS>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
-                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order) {
-    trace_body<false, AUXM, REC, MIXED, EXTRAS>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order);
+                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width) {
+    trace_body<false, AUXM, REC, MIXED, EXTRAS>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width);
 }
 template <int AUXM, bool REC, bool MIXED, bool DET>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
 void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
-                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order) {
-    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order);
+                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width) {
+    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width);
 }
 
 // Closing kernels of the deterministic mode: fixed point -> fp32, added to the caller's (zero-filled) tensors.
@@ -2059,22 +2079,29 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
     }
     // The per-lane walk is built into the kernels used where waves of unrelated rays are to be expected:
     // reflection bounces and ray lists (thin grids).  Image-shaped grids traced to depth 0 get the pure packet kernels.
+    // Order of the blocks of an image grid (trace_body): column strips put vertical neighbours on one XCD.  Measured
+    // forward, strips of 8 / 16 / 24 blocks / row-major: 8.12 / 8.20 / 8.53 / 8.48 ms on 120 x 68 blocks (1080p, 1M
+    // surfels), but 4.68 / 4.37 / 4.19 / 4.28 ms on 50 x 50 blocks (a sphere in front of an empty background): with only
+    // two or three rounds of workgroups on the chip the order decides more about the last round than about the caches.
+    // The backward trace gains 1 to 3 % from strips of 8 on every grid measured.
+    uint32_t strip = 0u;
+    if (t.th_log2 != 0) strip = BWD ? (uint32_t)DST_STRIP_BWD : (n_blocks >= kStripMinBlocks ? (uint32_t)DST_STRIP_FWD : 0u);
     const bool mixed = p.max_trace_depth > 0 || t.th_log2 < 3;
     const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
 #define DST_LAUNCH_M(AUX, MIXED)                                                                                   \
     do {                                                                                                           \
         if (BWD && det)                                                                                            \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, true>), grid, block, 0, stream, p, acc,      \
-                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                 \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                 \
         else if (BWD)                                                                                              \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, false>), grid, block, 0, stream, p, acc,     \
-                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                 \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                 \
         else if (p.flags != 0u)                                                                                    \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, true>), grid, block, 0, stream, p, acc, t.tw_log2,    \
-                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                            \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                            \
         else                                                                                                       \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, false>), grid, block, 0, stream, p, acc, t.tw_log2,   \
-                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order);                            \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                            \
     } while (0)
 #define DST_LAUNCH(AUX)                                                                                            \
     do {                                                                                                           \
