@@ -190,9 +190,9 @@ def main():
     mixed = "true" if (depth > 0 or H < 8) else "false"   # kernels with the per-lane walk built in
     per_kernel = {"forward": roofline_of("forward", "k_trace_fwd<%d,true,%s,false>" % (aux_max, mixed), A_fwd, fwd_ms),
                   "backward": roofline_of("backward", "k_trace_bwd<%d,true,false,false>" % aux_max, A_bwd, bwd_ms)}
-    # the dominant kernel is the slower one (the two are within a few per cent of each other on this workload,
-    # so both are reported under `roofline_kernels`)
-    roofline = per_kernel["backward" if bwd_ms >= fwd_ms else "forward"]
+    # The two kernels take about the same time on this workload, so "the slower one" flips from run to run.  `roofline`
+    # is the one further from its bound (the lower fraction: the one to work on); both are under `roofline_kernels`.
+    roofline = min(per_kernel.values(), key=lambda r: r["frac"])
 
     result = {
         "metric": "rays/s fwd+bwd at 1M surfels 1080p" if args.workload == "config3" else "rays/s fwd+bwd",
