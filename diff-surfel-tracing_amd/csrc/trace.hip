@@ -909,6 +909,32 @@ __device__ __forceinline__ void wave_add_grouped(float *base, unsigned long long
     if (on) add(key, v);
 }
 
+// The blending weights of an image wave (forward, training): a wave composites the same two hundred or so surfels over
+// and over (64 neighbouring rays, some 37 hits each), so their weights are first summed in a small hash table in LDS
+// (surfel id -> running sum, LDS atomics) and go to memory once per surfel and wave when the wave ends - a sixteenth of
+// the global atomics.  A surfel that finds no slot within a few probes adds straight to memory.
+constexpr int kWetSlotsLog2 = 8, kWetSlots = 1 << kWetSlotsLog2, kWetProbes = 4;
+__device__ __forceinline__ void wet_add(uint32_t *keys, float *vals, float *a_weights, bool on, uint32_t g, float w) {
+    if (!on) return;
+    uint32_t slot = (g * 2654435761u) >> (32 - kWetSlotsLog2);
+#pragma unroll 1
+    for (int probe = 0; probe < kWetProbes; ++probe) {
+        uint32_t k = __hip_atomic_load(keys + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (k == 0xFFFFFFFFu) {
+            uint32_t expected = 0xFFFFFFFFu;
+            __hip_atomic_compare_exchange_strong(keys + slot, &expected, g, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_WORKGROUP);
+            k = expected == 0xFFFFFFFFu ? g : expected;
+        }
+        if (k == g) {
+            __hip_atomic_fetch_add(vals + slot, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            return;
+        }
+        slot = (slot + 1u) & (uint32_t)(kWetSlots - 1);
+    }
+    aadd(a_weights + g, w);
+}
+
 // Find or claim the table row of surfel g; -1 if none is free within a few probes.  keys[rows] counts the
 // rows claimed since the table was last emptied.
 template <int ROWS_LOG2>
@@ -1601,9 +1627,11 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                 Tp = Tn;
             } while (false);
             if (REC && BWD) fetch_geometry(want_next);
-            if (!BWD && p.training && p.a_weights != nullptr)
-                wave_add_grouped(p.a_weights, (DET && (p.flags & DST_FLAG_DETERMINISTIC)) ? p.det_workspace : nullptr, did,
-                                 (uint32_t)g, w);
+            if (!BWD && p.training && p.a_weights != nullptr) {
+                if (!MIXED && !DET) wet_add(tab_keys, tab_rows, p.a_weights, did, (uint32_t)g, w);   // the wave's LDS table
+                else wave_add_grouped(p.a_weights, (DET && (p.flags & DST_FLAG_DETERMINISTIC)) ? p.det_workspace : nullptr, did,
+                                      (uint32_t)g, w);
+            }
             // ---- phase 2 (whole wave, backward only): gradients of the hits composited above -----------
             if (BWD && wave_ballot(did) != 0ull) {
                 GradSink<AUXM, DET> sink;
@@ -1687,6 +1715,19 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     __shared__ float s_stage[BWD ? kWavesPerBlock * kStageWords : 1];
     uint32_t *tab_keys = s_keys;
     float *tab_rows = s_rows;
+    // forward of an image at depth 0: the wave's table of blending weights (wet_add; in the kernels that carry the
+    // per-lane walk it measured no gain and would take the LDS to the limit of 16 waves per CU)
+    constexpr bool WET = !BWD && !MIXED && !DET;
+    __shared__ uint32_t s_wet_keys[WET ? kFwdWavesPerBlock * kWetSlots : 1];
+    __shared__ float s_wet_vals[WET ? kFwdWavesPerBlock * kWetSlots : 1];
+    uint32_t *const wet_keys = s_wet_keys + (WET ? (threadIdx.x / DST_WAVE) * kWetSlots : 0);
+    float *const wet_vals = s_wet_vals + (WET ? (threadIdx.x / DST_WAVE) * kWetSlots : 0);
+    if (WET) {   // (a wave's LDS accesses keep their order: no barrier between this and the first use)
+        for (int e = threadIdx.x % DST_WAVE; e < kWetSlots; e += DST_WAVE) {
+            wet_keys[e] = 0xFFFFFFFFu;
+            wet_vals[e] = 0.f;
+        }
+    }
     // Backward with a hit record: the launcher starts the replaying kernel and the re-tracing kernel one after
     // the other, and word 0 of the record (blocks the forward trace asked for) decides on the device which of
     // the two does the work: the host never has to wait for the forward trace to learn whether its record is complete.
@@ -1774,7 +1815,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             F3 dist_acc = f3(0, 0, 0);
-            walk_bounce<false, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, nullptr, nullptr, nullptr, rv, i, dist_acc WS_ARG);
+            walk_bounce<false, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, WET ? wet_keys : nullptr, WET ? wet_vals : nullptr, nullptr, rv, i, dist_acc WS_ARG);
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -1830,6 +1871,13 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             p.out_rgb[3 * r + 0] = out_rgb[0];
             p.out_rgb[3 * r + 1] = out_rgb[1];
             p.out_rgb[3 * r + 2] = out_rgb[2];
+        }
+        if (WET && p.training && p.a_weights != nullptr) {   // the wave's blending weights: one addition per surfel
+            for (int e = (int)lane; e < kWetSlots; e += DST_WAVE) {
+                const uint32_t k = wet_keys[e];
+                const float v = wet_vals[e];
+                if (k != 0xFFFFFFFFu && v != 0.f) aadd(p.a_weights + k, v);
+            }
         }
         if (p.counters != nullptr) {
             uint32_t a = wave_sum(n_proc), b = wave_sum(n_con);
