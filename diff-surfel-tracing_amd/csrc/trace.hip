@@ -798,7 +798,8 @@ __device__ __forceinline__ void aadd(float *p, float v) { unsafeAtomicAdd(p, v);
 // global memory once per surfel and block when the block ends.  A surfel that finds no free row within a
 // few probes goes straight to global atomics, so the table can never be wrong, only less effective.
 #ifndef DST_TABLE_FLUSH_NUM
-#define DST_TABLE_FLUSH_NUM 6   // the table is emptied between rounds once this many eighths of its rows are in use
+#define DST_TABLE_FLUSH_NUM 3   // the table is emptied between rounds once this many eighths of its rows are in use
+                                // (measured 1..6: a fuller table sends more hits past it, straight to memory)
 #endif
 #ifndef DST_TABLE_ROWS_LOG2
 #define DST_TABLE_ROWS_LOG2 7
