@@ -106,6 +106,8 @@ struct dst_ctx {
     // ordering of ray lists (thin ray grids): sort keys / ray numbers ping-pong and radix histograms, grow-only
     uint32_t *ray_keys[2] = {nullptr, nullptr}, *ray_vals[2] = {nullptr, nullptr}, *ray_hist = nullptr;
     uint32_t ray_capacity = 0;
+    uint32_t *block_order = nullptr;   // dispatch order of a replaying backward trace (longest blocks first), grow-only
+    uint32_t block_order_capacity = 0;
     DstBounds *bounds = nullptr;       // device
     DstBounds *bounds_host = nullptr;  // pinned host copy
     float scene_lo[3] = {0, 0, 0}, scene_hi[3] = {0, 0, 0}, max_abs = 0;

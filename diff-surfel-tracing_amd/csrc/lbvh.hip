@@ -835,6 +835,8 @@ void dst_lbvh_free(dst_ctx *ctx) {
     rel(ctx->ray_vals[0]);
     rel(ctx->ray_vals[1]);
     rel(ctx->ray_hist);
+    rel(ctx->block_order);
+    ctx->block_order_capacity = 0;
     ctx->ray_capacity = 0;
     ctx->capacity = 0;
     ctx->built = false;

@@ -33,6 +33,8 @@ constexpr int kFwdWavesPerBlock = DST_FWD_WPB;   // 1 or kWavesPerBlock
 #ifndef DST_STRIP_BWD
 #define DST_STRIP_BWD 8
 #endif
+constexpr uint32_t kOrderMinBlocks = 1536;   // replay: blocks are taken longest first on grids of at least two rounds of blocks
+                                             // (768 fit the chip at once; below that the order kernel costs more than it saves)
 constexpr uint32_t kStripMinBlocks = 4096;   // forward: strips only for grids of at least this many blocks (see launch())
 
 __device__ const float SH0 = 0.28209479177387814f;
@@ -1324,10 +1326,12 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
 // them instead of walking the BVH again.  Layout of the caller's buffer, in 8-byte words:
 //   [0] blocks requested so far (the forward kernel counts on past the capacity, which is how overflow shows)
 //   [1] chains that a replay found broken (stays 0 for a record written by a forward trace with a zeroed header)
-//   [2 ...) directory: one uint32 per (wave, bounce slot) = 1 + first block of that wave's bounce, 0 = none
+//   [2 ...) directory: one uint32 per (wave, bounce slot): low 26 bits = 1 + first block of that wave's bounce (0 =
+//           none), high 6 bits = the number of chunks the wave stored for that bounce (what its replay will cost)
 //   then `capacity` blocks of kRecBlockWords words: 16x64 entries ([slot][lane]), 64 uint32 counts, next+1, and
 //   the colour of every composited hit as the forward evaluated it ([slot][channel][lane] floats; a channel clamped
 //   at zero is stored as -0): the replay then neither gathers nor evaluates the 48 SH coefficients per hit again.
+constexpr uint32_t kRecDirBlockBits = 26, kRecDirBlockMask = (1u << kRecDirBlockBits) - 1u;
 constexpr uint32_t kRecColourWord = kChunk * DST_WAVE + DST_WAVE / 2 + 8;   // first word of the colours
 constexpr uint32_t kRecBlockWords = kRecColourWord + kChunk * 3 * DST_WAVE / 2;
 struct RecView {
@@ -1344,7 +1348,7 @@ __device__ __forceinline__ float *rec_store(const RecView &rv, int bounce, uint3
     uint32_t blk = 0;
     if (lane == 0) blk = (uint32_t)atomicAdd((unsigned long long *)rv.base, 1ull);
     blk = __builtin_amdgcn_readfirstlane(blk);
-    if (blk >= rv.capacity) return nullptr;   // too small: the host sees the count and the backward pass re-traces
+    if (blk >= rv.capacity || blk >= kRecDirBlockMask) return nullptr;   // too small: the host sees the count and the backward pass re-traces
     uint64_t *b = rv.blocks + (size_t)blk * kRecBlockWords;
 #pragma unroll
     for (int k = 0; k < kChunk; ++k) __builtin_nontemporal_store(buf.e[k], b + k * DST_WAVE + lane);
@@ -1445,7 +1449,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     wl.out = wl.in + (RESUME ? kListCap : 0);
     wl.n_in = kListFresh;
     wl.record = false;
-    uint32_t rec_pos = (REC && BWD) ? rv.dir[bounce] : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
+    uint32_t rec_pos = (REC && BWD) ? (rv.dir[bounce] & kRecDirBlockMask) : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
+    uint32_t rec_chunks = 0u;   // forward with a record: chunks stored for this bounce
     for (;;) {
         // Backward: the four waves of the block take their chunks in step, so that between two rounds nobody
         // touches the gradient table and it can be emptied when it fills up.
@@ -1473,7 +1478,10 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         } else {
             kbuf_reset(buf);
             packet_knn<MIXED, SHELF, RESUME>(acc, max_abs, ot, rd, live, buf, cnt, as_packet, wl, wave_lds WSP);
-            if (REC && !BWD) rec_colours = rec_store(rv, bounce, rec_pos, buf, cnt);
+            if (REC && !BWD) {
+                rec_colours = rec_store(rv, bounce, rec_pos, buf, cnt);
+                rec_chunks += rec_colours != nullptr ? 1u : 0u;
+            }
         }
         STAT(unsigned long long c1 = __builtin_readcyclecounter(); ws.t_trav += c1 - c0;)
         int here = 0;
@@ -1674,6 +1682,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         }
     }
+    if (REC && !BWD && rec_chunks != 0u && __lane_id() == 0u)   // the replay's cost of this wave and bounce, for its launcher
+        rv.dir[bounce] = (rv.dir[bounce] & kRecDirBlockMask) | (min(rec_chunks, 63u) << kRecDirBlockBits);
     STAT(if (BWD) { ws.nodes += last_sh.t_alg; ws.leaves += last_sh.t_sh; })
     if (BWD && p.colors_precomp == nullptr && last_sh.any)
         g_rd = sh_direction_gradient(p.D, p.shs + (size_t)last_sh.g * p.M * 3, rd, last_sh.gc);
@@ -1704,10 +1714,68 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
     return v;
 }
 
+// Position j in the dispatch order of an image grid -> block (bx, by): column strips `strip` blocks wide, row by row
+// inside a strip (strip 0 or a ray list: row-major).  See trace_body for why.
+__device__ __forceinline__ void block_of_position(uint32_t j, uint32_t btiles_x, uint32_t rows, uint32_t strip_width,
+                                                  bool image, uint32_t &bx, uint32_t &by) {
+    bx = j % btiles_x;
+    by = j / btiles_x;
+    if (strip_width != 0u && image) {
+        const uint32_t per_strip = strip_width * rows, strip = j / per_strip, r = j % per_strip;
+        if (strip * strip_width < btiles_x) {   // (positions past the grid keep the row-major numbers: their blocks leave)
+            const uint32_t w = min(strip_width, btiles_x - strip * strip_width);
+            bx = strip * strip_width + r % w;
+            by = r / w;
+        }
+    }
+}
+
+// Order of the blocks of a replaying backward trace: longest first.  The forward trace left in the record's directory
+// how many chunks every wave stored (what its replay costs); a block takes as long as the longest of its four waves
+// (they take their chunks in step).  With the long blocks first, the chip runs out of work with short blocks, not
+// with one long block per CU still going.  One workgroup: a counting sort over 64 cost classes, positions taken
+// 1024 at a time so that blocks of equal cost keep their neighbourhood.
+__global__ __launch_bounds__(1024) void k_block_order(const uint32_t *__restrict__ dir, uint32_t slots, uint32_t btiles_x,
+                                                     uint32_t rows, uint32_t strip_width, int image, uint32_t n_blocks,
+                                                     uint32_t *__restrict__ order) {
+    __shared__ uint32_t s_count[64], s_base[64];
+    auto cost_class = [&](uint32_t j) -> uint32_t {   // 0 = the most expensive
+        uint32_t bx, by;
+        block_of_position(j, btiles_x, rows, strip_width, image != 0, bx, by);
+        if (by >= rows) return 63u;
+        const uint32_t *d = dir + (size_t)(by * btiles_x + bx) * kWavesPerBlock * slots;
+        uint32_t worst = 0u;
+        for (uint32_t w = 0; w < (uint32_t)kWavesPerBlock; ++w) {
+            uint32_t sum = 0u;
+            for (uint32_t k = 0; k < slots; ++k) sum += d[w * slots + k] >> kRecDirBlockBits;
+            worst = max(worst, sum);
+        }
+        return 63u - min(worst, 63u);
+    };
+    if (threadIdx.x < 64) s_count[threadIdx.x] = 0u;
+    __syncthreads();
+    for (uint32_t j = threadIdx.x; j < n_blocks; j += blockDim.x) atomicAdd(&s_count[cost_class(j)], 1u);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t run = 0u;
+        for (int c = 0; c < 64; ++c) {
+            s_base[c] = run;
+            run += s_count[c];
+        }
+    }
+    __syncthreads();
+    for (uint32_t base = 0; base < n_blocks; base += blockDim.x) {   // in order, 1024 positions at a time
+        const uint32_t j = base + threadIdx.x;
+        if (j < n_blocks) order[atomicAdd(&s_base[cost_class(j)], 1u)] = j;
+        __syncthreads();
+    }
+}
+
 template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x,
-                                           const uint32_t *__restrict__ ray_order, uint32_t strip_width) {
+                                           const uint32_t *__restrict__ ray_order, uint32_t strip_width,
+                                           const uint32_t *__restrict__ block_order) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     constexpr int kTableRows = RowLayout<AUXM>::rows;
@@ -1758,17 +1826,9 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     // vertical neighbours and meet the same BVH nodes in that XCD's own L2 (row-major order over a 120-block-wide image
     // gave an XCD blocks eight columns apart: forward 8.5 -> 8.1 ms on the 1080p room scene).  The last strip may be
     // narrower; its blocks are spread over all XCDs like the others.  The launcher chooses the width (launch()).
-    const uint32_t kStrip = strip_width;   // 0: row-major
-    uint32_t bx = bid % btiles_x, by = bid / btiles_x;
-    if (kStrip != 0u && th_log2 != 0) {
-        const uint32_t rows = (tiles_y + 1u) / 2u, per_strip = kStrip * rows;
-        const uint32_t strip = bid / per_strip, r = bid % per_strip;
-        if (strip * kStrip < btiles_x) {   // (blocks past the grid keep the row-major numbers and leave below)
-            const uint32_t w = min(kStrip, btiles_x - strip * kStrip);
-            bx = strip * kStrip + r % w;
-            by = r / w;
-        }
-    }
+    if (BWD && block_order != nullptr) bid = block_order[bid];   // replay: the longest blocks first (k_block_order)
+    uint32_t bx, by;
+    block_of_position(bid, btiles_x, (tiles_y + 1u) / 2u, strip_width, th_log2 != 0, bx, by);
     const bool flat = th_log2 == 0;   // a ray list: tiles of 1x64 rays, a block = four consecutive tiles
     if (flat ? by >= 1u : 2u * by >= tiles_y) return;   // padding of the forward grid (whole blocks)
     RecView rv = {nullptr, nullptr, nullptr, 0u};
@@ -2005,13 +2065,14 @@ template <int AUXM, bool REC, bool MIXED, bool EXTRAS>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width) {
-    trace_body<false, AUXM, REC, MIXED, EXTRAS>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width);
+    trace_body<false, AUXM, REC, MIXED, EXTRAS>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, nullptr);
 }
 template <int AUXM, bool REC, bool MIXED, bool DET>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
 void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
-                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width) {
-    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width);
+                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width,
+                 const uint32_t *block_order) {
+    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, block_order);
 }
 
 // Closing kernels of the deterministic mode: fixed point -> fp32, added to the caller's (zero-filled) tensors.
@@ -2119,7 +2180,8 @@ TileGrid tile_grid(int H, int W) {
 }
 
 template <bool BWD, bool REC>
-void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, const uint32_t *ray_order, hipStream_t stream) {
+void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, const uint32_t *ray_order, hipStream_t stream,
+            const uint32_t *block_order = nullptr) {
     const uint32_t n_blocks = t.btiles_x * t.btiles_y;
     dim3 grid(n_blocks), block(kWavesPerBlock * DST_WAVE);
     if (!BWD && kFwdWavesPerBlock == 1) {
@@ -2141,10 +2203,10 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
     do {                                                                                                           \
         if (BWD && det)                                                                                            \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, true>), grid, block, 0, stream, p, acc,      \
-                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                 \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip, block_order);    \
         else if (BWD)                                                                                              \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, false>), grid, block, 0, stream, p, acc,     \
-                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                 \
+                               t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip, block_order);    \
         else if (p.flags != 0u)                                                                                    \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, true>), grid, block, 0, stream, p, acc, t.tw_log2,    \
                                t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                            \
@@ -2234,7 +2296,24 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
     const bool rec = p.hit_record != nullptr;
     const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
     if (backward) {
-        if (rec) launch<true, true>(p, acc, t, ray_order, stream);   // does the work if the record is complete,
+        const uint32_t n_blocks = t.btiles_x * t.btiles_y;
+        if (rec && n_blocks < kOrderMinBlocks) {
+            launch<true, true>(p, acc, t, ray_order, stream);
+        } else if (rec) {
+            // the replay takes its blocks longest first (the forward left every wave's chunk count in the record)
+            if (n_blocks > ctx->block_order_capacity) {
+                if (ctx->block_order) (void)hipFree(ctx->block_order);
+                ctx->block_order = nullptr;
+                ctx->block_order_capacity = 0;
+                DST_HIP(ctx, hipMalloc((void **)&ctx->block_order, sizeof(uint32_t) * n_blocks));
+                ctx->block_order_capacity = n_blocks;
+            }
+            const uint32_t strip = t.th_log2 != 0 ? (uint32_t)DST_STRIP_BWD : 0u;
+            hipLaunchKernelGGL(k_block_order, dim3(1), dim3(1024), 0, stream,
+                               reinterpret_cast<const uint32_t *>(p.hit_record + 2), (uint32_t)p.mtd_alloc + 1u, t.btiles_x,
+                               t.btiles_y, strip, t.th_log2 != 0 ? 1 : 0, n_blocks, ctx->block_order);
+            launch<true, true>(p, acc, t, ray_order, stream, ctx->block_order);   // does the work if the record is complete,
+        }
         launch<true, false>(p, acc, t, ray_order, stream);           // else this one does (it returns at once otherwise)
         const dim3 grid(2048), block(256);
         if (det) {
