@@ -1752,9 +1752,15 @@ __global__ __launch_bounds__(1024) void k_block_order(const uint32_t *__restrict
         }
         return 63u - min(worst, 63u);
     };
+    constexpr uint32_t kKept = 32768;   // classes of the first pass kept in LDS for the second (grids up to this size)
+    __shared__ uint8_t s_class[kKept];
     if (threadIdx.x < 64) s_count[threadIdx.x] = 0u;
     __syncthreads();
-    for (uint32_t j = threadIdx.x; j < n_blocks; j += blockDim.x) atomicAdd(&s_count[cost_class(j)], 1u);
+    for (uint32_t j = threadIdx.x; j < n_blocks; j += blockDim.x) {
+        const uint32_t c = cost_class(j);
+        if (j < kKept) s_class[j] = (uint8_t)c;
+        atomicAdd(&s_count[c], 1u);
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t run = 0u;
@@ -1766,7 +1772,7 @@ __global__ __launch_bounds__(1024) void k_block_order(const uint32_t *__restrict
     __syncthreads();
     for (uint32_t base = 0; base < n_blocks; base += blockDim.x) {   // in order, 1024 positions at a time
         const uint32_t j = base + threadIdx.x;
-        if (j < n_blocks) order[atomicAdd(&s_base[cost_class(j)], 1u)] = j;
+        if (j < n_blocks) order[atomicAdd(&s_base[j < kKept ? (uint32_t)s_class[j] : cost_class(j)], 1u)] = j;
         __syncthreads();
     }
 }

@@ -93,7 +93,7 @@ typedef struct DstParams {
      * call.  Word 0 then holds the number of blocks the forward trace asked for.  If that exceeds
      * hit_record_blocks the record is incomplete: the backward trace sees this ON THE DEVICE and walks the BVH
      * again instead (the host need not look at the record between the two calls; it may read word 0 later to
-     * size the next record).  Word 1 counts chains a replay found broken: it stays 0 unless the buffer was
+     * size the next record; at most 2^26 - 1 blocks of a record are used).  Word 1 counts chains a replay found broken: it stays 0 unless the buffer was
      * not written by a forward trace with the same grid, depth and a zeroed header. */
     uint64_t *hit_record;
     uint32_t hit_record_blocks;
