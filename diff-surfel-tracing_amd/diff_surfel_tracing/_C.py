@@ -254,7 +254,9 @@ class OptiXStateWrapper:
         self._record_pool.append(rec.words)
         rec.words = None
         if not self._record_fixed and len(self._record_pool) > self.RECORD_POOL_SIZE:
-            self._record_pool.remove(min(self._record_pool, key=lambda t: t.numel()))
+            # by identity: list.remove() would compare tensors element-wise
+            smallest = min(self._record_pool, key=lambda t: t.numel())
+            self._record_pool = [t for t in self._record_pool if t is not smallest]
 
     def accel_info(self):
         info = DstAccelInfo()

@@ -187,3 +187,26 @@ def test_no_hit_record_is_made_when_no_backward_can_follow(monkeypatch):
     plain[6] = torch.zeros(P, 3)       # no input asks for a gradient
     dst.trace_surfels(*plain)
     assert ctx2.acquired == 0
+
+
+def test_record_pool_takes_back_records_of_any_size():
+    """The pool of hit-record storages keeps the largest RECORD_POOL_SIZE tensors; returning one more, of any size
+    (training at several resolutions does that), drops the smallest and must not compare tensors by value."""
+    from diff_surfel_tracing import _C
+
+    class _Rec:
+        def __init__(self, n):
+            self.words = torch.zeros(n, dtype=torch.int64)
+
+    pool = _C.OptiXStateWrapper.__new__(_C.OptiXStateWrapper)   # no device: only the pool's bookkeeping is used
+    pool._record_pool, pool._record_fixed = [], False
+    sizes = [7, 3, 9, 3, 5, 11, 2, 9]
+    recs = [_Rec(n) for n in sizes]
+    for r in recs:
+        pool.release_record(r)
+        assert r.words is None
+    kept = sorted(t.numel() for t in pool._record_pool)
+    assert kept == sorted(sizes)[-_C.OptiXStateWrapper.RECORD_POOL_SIZE:]
+    pool.release_record(recs[0])    # a record already handed back is ignored
+    pool.release_record(None)
+    assert len(pool._record_pool) == _C.OptiXStateWrapper.RECORD_POOL_SIZE

@@ -108,6 +108,17 @@ def test_ragged_image_sizes(oracle, tracer):
         check_case(oracle, tracer, sc, *S.rays_cube(H, W))
 
 
+def test_many_image_sizes_through_one_context(oracle):
+    """Training at changing resolutions: every backward call hands its hit record back to the context's pool, which
+    then holds storages of many sizes and drops the smallest ones."""
+    import diff_surfel_tracing as dst
+    own = dst.SurfelTracer()
+    sc = S.scene_cube(P=1500, seed=6)
+    for H, W in ((8, 8), (40, 24), (16, 16), (72, 64), (24, 8), (56, 56), (8, 16), (32, 32), (64, 72)):
+        check_case(oracle, own, sc, *S.rays_cube(H, W, view=H % 3))
+    assert 1 <= len(own.optix_context._record_pool) <= own.optix_context.RECORD_POOL_SIZE
+
+
 @pytest.mark.parametrize("P", [1, 2, 3, 5])
 def test_tiny_scenes(oracle, tracer, P):
     sc = S.scene_cube(P=P, seed=P)
