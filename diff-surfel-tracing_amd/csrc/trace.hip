@@ -1204,14 +1204,8 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
 
     // triangle that was hit, with its corner coordinates in splat units (backward.cu:583-602)
     const float *V = p.vertices + (size_t)g * 12;
-    F3 v1, v2, v3, h1, h2, h3;
-    if ((pidx & 1u) == 0u) {
-        v1 = ld3(V); v2 = ld3(V + 3); v3 = ld3(V + 6);
-        h1 = f3(-3.f, 3.f, 3.f); h2 = f3(-3.f, -3.f, 3.f); h3 = f3(3.f, 3.f, 3.f);
-    } else {
-        v1 = ld3(V + 3); v2 = ld3(V + 6); v3 = ld3(V + 9);
-        h1 = f3(-3.f, -3.f, 3.f); h2 = f3(3.f, 3.f, 3.f); h3 = f3(3.f, -3.f, 3.f);
-    }
+    const bool second = (pidx & 1u) != 0u;
+    const F3 v1 = ld3(second ? V + 3 : V), v2 = ld3(second ? V + 6 : V + 3), v3 = ld3(second ? V + 9 : V + 6);
     const float k = g_G * pc;
     const float gu = k * -G * u, gv = k * -G * v;
     F3 gR[3];
@@ -1228,20 +1222,27 @@ __device__ __forceinline__ void hit_backward(const DstParams &p, const BounceIn<
     const F3 c = v1 - ro;
     const float pp = dot(n, c), q = dot(n, rd), inv_q = __builtin_amdgcn_rcpf(q);
     const F3 g_n = (c - (pp * inv_q) * rd) * inv_q;
-    const F3 g_v1 = g_d * cross(v2 - v3, g_n) + (g_d * inv_q) * n;
-    const F3 g_v2 = g_d * cross(v3 - v1, g_n);
-    const F3 g_v3 = g_d * cross(v1 - v2, g_n);
     if (did) {
         g_ro = g_ro + (g_xyz + (-g_d * inv_q) * n);
         g_rd = g_rd + (g_xyz * dpt + ((g_d * -pp) * (inv_q * inv_q)) * n);
     }
-    const F3 su = h1.x * g_v1 + h2.x * g_v2 + h3.x * g_v3;
-    const F3 sv = h1.y * g_v1 + h2.y * g_v2 + h3.y * g_v3;
+    // The corner gradients (backward.cu:583-602) are g_v1 = g_d (v2-v3) x g_n + (g_d/q) n, g_v2 = g_d (v3-v1) x g_n,
+    // g_v3 = g_d (v1-v2) x g_n, and the corners sit at (+-3, +-3) splat units.  Their sums with those weights are
+    // taken on the edge vectors first, where they collapse to one edge each: the three cross products nearly
+    // cancel for a long thin quad, and summed after the fact they leave mostly rounding.
+    //   sum of the corners' gradients          = (g_d/q) n
+    //   weighted by the corners' u coordinates = g_d 6 a x g_n + hu (g_d/q) n
+    //   weighted by the corners' v coordinates = g_d 6 b x g_n + hv (g_d/q) n
+    // with a = v1-v2, b = v1-v3, (hu,hv) = (-3,3) for the first triangle; a = v3-v2, b = v3-v1, (-3,-3) for the second.
+    const F3 g_c = (g_d * inv_q) * n;
+    const F3 ea = second ? v3 - v2 : v1 - v2, eb = second ? v3 - v1 : v1 - v3;
+    const F3 su = (6.f * g_d) * cross(ea, g_n) - 3.f * g_c;
+    const F3 sv = (6.f * g_d) * cross(eb, g_n) + (second ? -3.f : 3.f) * g_c;
     gR[0] = gR[0] + sx * su;
     gR[1] = gR[1] + sy * sv;
     g_sx += dot(R[0], su);
     g_sy += dot(R[1], sv);
-    g_mean = g_mean + (g_v1 + g_v2 + g_v3);
+    g_mean = g_mean + g_c;
     // rotation: vjp of quat_rows without the normalisation Jacobian (auxiliary.h:433-477)
     float g_rot[4];
     {
