@@ -85,3 +85,35 @@ def test_config4_room_500k_720p_depth2_forward_and_backward(oracle, tracer):
     assert (np.abs(slots[:, :, 2, 3:6]).sum(-1) > 0).mean() > 0.3     # the third bounce is traced for many rays
     acc = out["acc"].astype(np.float64)
     assert (acc >= 0).all() and (acc <= 1).all()
+
+
+@pytest.mark.parametrize("P,H,W,depth,aux", [(1000000, 2160, 3840, 0, 0), (300000, 1080, 1920, 2, 8)])
+def test_a_larger_image_equals_its_quadrants_traced_on_their_own(tracer, P, H, W, depth, aux):
+    """A size the oracle cannot reach in seconds (8.3M rays), held against a property that does not depend on size:
+    no per-ray result depends on which rays share a wave, an image or a launch, so the image and its four quadrants
+    must agree bit for bit in every per-ray output, and the quadrants' per-surfel gradients must add up to the image's."""
+    sc = S.scene_room(P=P, seed=3, aux=aux)
+    kw = {}
+    if depth:
+        sc["others_precomp"][:, 0] = sc["others_precomp"][:, 0] * 0.8 + 0.1
+        kw = dict(max_trace_depth=depth, specular_threshold=0.1)
+    o, d = S.rays_room(H, W)
+    ug = upstream(H, W, max(aux, 2))
+    full, gfull = gpu_trace(tracer, sc, o, d, upstream=ug, **kw)
+    assert np.isfinite(full["rgb"]).all() and full["acc"].mean() > 0.5
+    hh, hw = H // 2, W // 2
+    total = None
+    for r0, c0 in ((0, 0), (0, hw), (hh, 0), (hh, hw)):
+        sl = (slice(r0, r0 + hh), slice(c0, c0 + hw))
+        part, gpart = gpu_trace(tracer, sc, o[sl].contiguous(), d[sl].contiguous(),
+                                upstream={k: v[sl].contiguous() for k, v in ug.items()}, build=False, **kw)
+        for k in ("rgb", "dpt", "acc", "norm", "aux", "mid"):
+            a = np.ascontiguousarray(full[k].reshape(H, W, -1)[sl])
+            assert np.array_equal(a.view(np.uint32), part[k].reshape(hh, hw, -1).view(np.uint32)), (k, r0, c0)
+        for k in ("ray_o", "ray_d"):
+            a, b = gfull[k][sl], gpart[k]
+            assert np.abs(a - b).max() <= 1e-5 * np.abs(b).max(), k
+        rest = {k: v.astype(np.float64) for k, v in gpart.items() if v is not None and k not in ("ray_o", "ray_d")}
+        total = rest if total is None else {k: total[k] + rest[k] for k in total}
+    for k, v in total.items():
+        assert_close_sum(gfull[k], v, GRAD_REL, k)
