@@ -169,6 +169,7 @@ int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info) {
     info->max_abs = ctx->max_abs;
     info->builds = ctx->builds;
     info->refits = ctx->refits;
+    info->key_levels = ctx->fine_keys ? 2u : 1u;
     return DST_OK;
 }
 

@@ -66,6 +66,8 @@ struct DstBounds {          // device-resident reduction targets, order-preservi
     uint32_t lo[3], hi[3];  // centroid bounds
     uint32_t max_abs;       // raw bits of a non-negative float: largest |coordinate| of any vertex
     uint32_t bad_topology;  // set by the quad set-up kernel
+    uint32_t equal_keys;    // neighbours in Morton order with equal keys, counted while the hierarchy is made
+    uint32_t max_depth;     // nodes above the deepest leaf (builds with two-level keys only)
 };
 
 // Device-side view of the acceleration structure handed to the trace kernels.
@@ -85,6 +87,8 @@ struct dst_ctx {
     // acceleration structure
     uint32_t n_leaves = 0;      // surfels in the current structure
     uint32_t capacity = 0;      // surfels the buffers can hold
+    bool fine_keys = false;     // builds sort two-level Morton keys (set when a build finds the one-level grid too coarse)
+    bool fine_keys_refused = false;   // a build with two-level keys came out too deep for the walks' stacks
     bool built = false;
     uint32_t built_vertices = 0;   // rows of the vertex buffer the stored quad ids were validated against
     bool canonical = false;        // the build's quads were rows 4g..4g+3 of the vertex buffer, in that order

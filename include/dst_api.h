@@ -133,6 +133,9 @@ typedef struct DstAccelInfo {
     float scene_lo[3], scene_hi[3]; /* bounds of the quad centroids used for the Morton grid */
     float max_abs;         /* largest |coordinate| of any vertex */
     uint32_t builds, refits;
+    uint32_t key_levels;   /* 1: the builds sort 30-bit Morton keys; 2: 60-bit keys in two levels, which a context goes
+                              over to, for good, when a build finds more than three quarters of the surfels sharing
+                              their cell of the 1024^3 grid with a neighbour (surfels far outside a compact scene) */
 } DstAccelInfo;
 
 /* Create / destroy the tracer state on the current HIP device.

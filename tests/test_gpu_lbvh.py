@@ -111,6 +111,73 @@ def test_duplicate_positions_give_a_bounded_tree(tracer):
     assert depth <= 44   # 30 key bits + 12 index bits
 
 
+def _with_far_surfels(sc, factor, k=5, seed=4):
+    """`k` surfels of the scene moved `factor` scene radii away (and grown by as much)."""
+    out = {n: t.clone() for n, t in sc.items()}
+    gen = torch.Generator().manual_seed(seed)
+    dirs = torch.nn.functional.normalize(torch.randn(k, 3, generator=gen), dim=-1)
+    out["means3D"][:k] = dirs * factor * float(sc["means3D"].abs().max())
+    out["scales"][:k] = sc["scales"][:k] * factor
+    out["vertices"], out["faces"] = S.get_triangles(out["means3D"], out["scales"], out["rotations"])
+    return out
+
+
+def test_surfels_far_outside_a_compact_scene_switch_the_builds_to_two_level_keys():
+    """A few surfels 2000 scene radii away stretch the 1024^3 Morton grid until the scene itself fills one cell: the
+    build notices (nearly all neighbours in Morton order share their cell), builds again with 60-bit keys in two
+    levels and keeps them for the context's later builds.  The structure obeys the same invariants either way."""
+    import diff_surfel_tracing as dst
+    own = dst.SurfelTracer()
+    sc = S.scene_cube(P=20000, seed=8)
+    own.build_acceleration_structure(sc["vertices"].cuda(), sc["faces"].cuda(), True)
+    info, *arrs = download(own)
+    assert info.key_levels == 1 and info.builds == 1
+    flat_depth = check_tree(info, *arrs, sc["vertices"].numpy())
+    far = _with_far_surfels(sc, 2000.0)
+    own.build_acceleration_structure(far["vertices"].cuda(), far["faces"].cuda(), True)
+    info, *arrs = download(own)
+    assert info.key_levels == 2 and info.builds == 2     # the abandoned one-level build is not counted
+    depth = check_tree(info, *arrs, far["vertices"].numpy())
+    assert depth <= flat_depth + 12                       # the scene's own levels, and a few for the far surfels
+    # refit on the two-level structure, then a rebuild of the compact scene: still two levels
+    moved = S.perturb_means(far, 1, frac=0.5, sigma=0.2)
+    own.build_acceleration_structure(moved["vertices"].cuda(), far["faces"].cuda(), False)
+    info, *arrs = download(own)
+    check_tree(info, *arrs, moved["vertices"].numpy())
+    own.build_acceleration_structure(sc["vertices"].cuda(), sc["faces"].cuda(), True)
+    info, *arrs = download(own)
+    assert info.key_levels == 2
+    assert check_tree(info, *arrs, sc["vertices"].numpy()) <= flat_depth + 2
+
+
+def test_two_level_keys_are_given_up_when_the_hierarchy_gets_too_deep():
+    """Sixty surfels that each peel one bit off the 60-bit key (one per axis and scale, down to a millionth of the
+    extent) in front of 4096 surfels at one point: with two-level keys the deepest leaf lies 72 nodes down, more than
+    the walks' stacks are sized for.  The build measures that and returns to one-level keys for good."""
+    import diff_surfel_tracing as dst
+    own = dst.SurfelTracer()
+    pts = [[0.0, 0.0, 0.0]] * 4096
+    for k in range(20):
+        for a in range(3):
+            p = [0.0, 0.0, 0.0]
+            p[a] = 1.2 * 2.0 ** -k
+            pts.append(p)
+    P = len(pts)
+    sc = S.scene_cube(P=P, seed=5)
+    sc["means3D"] = torch.tensor(pts, dtype=torch.float32)
+    sc["scales"] = torch.full((P, 2), 1e-8)
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    own.build_acceleration_structure(sc["vertices"].cuda(), sc["faces"].cuda(), True)
+    info, *arrs = download(own)
+    assert info.key_levels == 1 and info.builds == 1
+    depth = check_tree(info, *arrs, sc["vertices"].numpy())
+    assert 40 <= depth < 62        # thirty peeled bits, then the 4096 + 30 surfels of the last cell
+    # the refusal holds: a scene that asks for two levels again is built with one
+    far = _with_far_surfels(S.scene_cube(P=3000, seed=8), 2000.0)
+    own.build_acceleration_structure(far["vertices"].cuda(), far["faces"].cuda(), True)
+    assert own.optix_context.accel_info().key_levels == 1
+
+
 def test_boundary_errors(tracer):
     import diff_surfel_tracing as dst
     sc = S.scene_cube(P=100, seed=0)

@@ -119,6 +119,29 @@ def test_many_image_sizes_through_one_context(oracle):
     assert 1 <= len(own.optix_context._record_pool) <= own.optix_context.RECORD_POOL_SIZE
 
 
+def test_surfels_far_outside_the_scene(oracle):
+    """Far surfels (some of them large and in view behind the scene) make the build go over to two-level Morton keys
+    and widen the padding of the box tests (it scales with the largest coordinate): results stay the oracle's."""
+    import diff_surfel_tracing as dst
+    from test_gpu_lbvh import _with_far_surfels
+    own = dst.SurfelTracer()
+    sc = _with_far_surfels(S.scene_cube(P=8000, seed=12, aux=2), 1500.0, k=6)
+    o, d = S.rays_cube(40, 48, view=1)
+    # two more far surfels straight behind the scene, facing the camera, so that rays reach them
+    back = -o[0, 0] / o[0, 0].norm()
+    for k, dist in ((6, 40.0), (7, 900.0)):
+        sc["means3D"][k] = back * dist
+        sc["scales"][k] = torch.tensor([0.1, 0.1]) * dist
+    nrm = (-back).expand(2, 3).clone()
+    from dst_scenes import _quat_from_normal
+    sc["rotations"][6:8] = _quat_from_normal(nrm, torch.Generator().manual_seed(0))
+    sc["opacities"][6:8] = 0.9
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    ref, _ = check_case(oracle, own, sc, o, d, bg=(0.1, 0.2, 0.3))
+    assert own.optix_context.accel_info().key_levels == 2
+    assert ref["wet"][6] > 0 and ref["wet"][7] > 0     # both far surfels are seen
+
+
 @pytest.mark.parametrize("P", [1, 2, 3, 5])
 def test_tiny_scenes(oracle, tracer, P):
     sc = S.scene_cube(P=P, seed=P)
