@@ -54,6 +54,9 @@ __global__ void k_fill_u32(uint32_t *p, uint32_t v, uint32_t n) {
     if (i < n) p[i] = v;
 }
 
+// The coordinate bound covers the finite coordinates: one corner at infinity must not void the bound of the others.
+__device__ __forceinline__ float finite_max(float m, float x) { return x < INFINITY ? fmaxf(m, x) : m; }
+
 // Largest |coordinate| of a block's quads -> bounds->max_abs: the waves meet in LDS, one atomic per block (atomics of
 // many waves to one word are served one by one).  Every thread of the block calls it.
 __device__ __forceinline__ void block_max_abs(float mabs, DstBounds *bounds) {
@@ -129,7 +132,7 @@ __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vert
             for (int a = 0; a < 3; ++a) {
                 lo[a] = fminf(lo[a], c[k][a]);
                 hi[a] = fmaxf(hi[a], c[k][a]);
-                mabs = fmaxf(mabs, fabsf(c[k][a]));
+                mabs = finite_max(mabs, fabsf(c[k][a]));
             }
         }
         float4 c4;
@@ -138,9 +141,10 @@ __global__ void k_quad_setup(const float *__restrict__ vertices, uint32_t n_vert
         c4.z = 0.5f * (lo[2] + hi[2]);
         c4.w = 0.f;
         centroids[g] = c4;
-        cen[0] = fminf(cen[0], c4.x); cenh[0] = fmaxf(cenh[0], c4.x);
-        cen[1] = fminf(cen[1], c4.y); cenh[1] = fmaxf(cenh[1], c4.y);
-        cen[2] = fminf(cen[2], c4.z); cenh[2] = fmaxf(cenh[2], c4.z);
+        // a centroid at infinity (or NaN) takes no part in the grid's extent; its key is clamped to the grid's edge
+        if (fabsf(c4.x) < INFINITY) { cen[0] = fminf(cen[0], c4.x); cenh[0] = fmaxf(cenh[0], c4.x); }
+        if (fabsf(c4.y) < INFINITY) { cen[1] = fminf(cen[1], c4.y); cenh[1] = fmaxf(cenh[1], c4.y); }
+        if (fabsf(c4.z) < INFINITY) { cen[2] = fminf(cen[2], c4.z); cenh[2] = fmaxf(cenh[2], c4.z); }
     }
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -632,7 +636,7 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
 #pragma unroll
         for (int k = 0; k < 4; ++k)
 #pragma unroll
-            for (int a = 0; a < 3; ++a) mabs = fmaxf(mabs, fabsf(c[k][a]));
+            for (int a = 0; a < 3; ++a) mabs = finite_max(mabs, fabsf(c[k][a]));
     }
     if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
     if (bounds != nullptr) block_max_abs(mabs, bounds);   // a refit: the coordinate bound of the moved quads
@@ -672,7 +676,7 @@ __global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const 
 #pragma unroll
             for (int a = 0; a < 3; ++a) {
                 c[k][a] = (m[a] + sa[k] * u[a]) + sb[k] * v[a];
-                mabs = fmaxf(mabs, fabsf(c[k][a]));
+                mabs = finite_max(mabs, fabsf(c[k][a]));
             }
         if (vertices_out != nullptr) {
             float4 *dst = reinterpret_cast<float4 *>(vertices_out + 12 * (size_t)g);   // 48 bytes per surfel

@@ -142,6 +142,26 @@ def test_surfels_far_outside_the_scene(oracle):
     assert ref["wet"][6] > 0 and ref["wet"][7] > 0     # both far surfels are seen
 
 
+def test_surfels_with_nan_and_infinite_parameters(oracle, tracer):
+    """A diverged optimisation leaves NaN and infinite means, scales and zero quaternions behind: such surfels are hit
+    by nothing, take no part in the grid's extent or the coordinate bound, and the others render as the oracle's."""
+    sc = S.scene_cube(P=6000, seed=31, aux=2)
+    r = torch.rand(6000, generator=torch.Generator().manual_seed(32))
+    sc["means3D"][r < 0.02, 0] = float("nan")
+    sc["means3D"][(r >= 0.02) & (r < 0.04), 1] = float("inf")
+    sc["means3D"][(r >= 0.04) & (r < 0.05), 2] = -float("inf")
+    sc["scales"][(r >= 0.05) & (r < 0.06), 0] = float("inf")
+    sc["scales"][(r >= 0.06) & (r < 0.07), 1] = float("nan")
+    sc["rotations"][(r >= 0.07) & (r < 0.08)] = 0.0
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    assert not torch.isfinite(sc["vertices"]).all()
+    ref, out = check_case(oracle, tracer, sc, *S.rays_cube(48, 48, view=2))
+    assert ref["n_con"].mean() > 3 and np.isfinite(out["rgb"]).all()
+    info = tracer.optix_context.accel_info()
+    assert np.isfinite(info.max_abs) and np.isfinite(list(info.scene_lo)).all() and np.isfinite(list(info.scene_hi)).all()
+    assert info.max_abs < 3.0 and max(info.scene_hi) < 2.0
+
+
 @pytest.mark.parametrize("P", [1, 2, 3, 5])
 def test_tiny_scenes(oracle, tracer, P):
     sc = S.scene_cube(P=P, seed=P)
