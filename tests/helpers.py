@@ -113,6 +113,20 @@ def assert_close_sum(a, b, rel, name, noise=None, max_noisy=0.02):
     assert noisy.mean() <= max_noisy, "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean())
 
 
+def assert_same_sums(a, b, rel, name):
+    """Two GPU results of the same sums whose float atomics ran in different orders (one image against its parts, one
+    call against the same call made another way).  Not the parity bar - that one has the oracle's noise estimate to
+    lean on: element-wise |a - b| <= rel * |b| + rel * (root mean square of the channel's nonzero entries)."""
+    assert a.shape == b.shape, (name, a.shape, b.shape)
+    a64 = np.asarray(a, np.float64).reshape(a.shape[0], -1)
+    b64 = np.asarray(b, np.float64).reshape(a.shape[0], -1)
+    rms = np.sqrt((b64 ** 2).sum(0) / np.maximum((b64 != 0).sum(0), 1))
+    err, tol = np.abs(a64 - b64), rel * np.abs(b64) + rel * rms[None, :]
+    bad = err > tol
+    assert not bad.any(), "%s: %d of %d elements off, worst %.2f of its tolerance" % (
+        name, int(bad.sum()), bad.size, float((err / np.maximum(tol, 1e-300)).max()))
+
+
 def assert_close_rays(a, b, rel, name, noise=None, max_noisy=0.02):
     """Per-ray gradients are plain stores (no atomics): element-wise |a - b| <= rel * |b| + rel/10 * (largest
     component of that ray's gradient) + NOISE_FACTOR * noise (see assert_close_sum)."""

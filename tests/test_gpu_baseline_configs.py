@@ -9,8 +9,8 @@ import pytest
 import torch
 
 import dst_scenes as S
-from helpers import (GRAD_REL, assert_close_sum, assert_forward_exact, assert_gradients, gpu_trace, oracle_scene,
-                     upstream)
+from helpers import (GRAD_REL, assert_close_sum, assert_forward_exact, assert_gradients, assert_same_sums, gpu_trace,
+                     oracle_scene, upstream)
 
 pytestmark = pytest.mark.gpu
 
@@ -116,4 +116,4 @@ def test_a_larger_image_equals_its_quadrants_traced_on_their_own(tracer, P, H, W
         rest = {k: v.astype(np.float64) for k, v in gpart.items() if v is not None and k not in ("ray_o", "ray_d")}
         total = rest if total is None else {k: total[k] + rest[k] for k in total}
     for k, v in total.items():
-        assert_close_sum(gfull[k], v, GRAD_REL, k)
+        assert_same_sums(gfull[k], v, GRAD_REL, k)

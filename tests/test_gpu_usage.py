@@ -2,13 +2,14 @@
 passes in any order, a second backward through a kept graph, inputs of which only some ask for gradients,
 non-contiguous views, a side stream, two contexts, gradient modes.  The reference is one call of each kind on
 its own (those are held against the oracle in test_gpu_parity.py): per-ray outputs must repeat bit for bit,
-atomically summed gradients within the parity tolerance."""
+atomically summed gradients within 1e-3 of the value plus 1e-3 of the channel's root mean square (two orders of
+float atomics)."""
 import numpy as np
 import pytest
 import torch
 
 import dst_scenes as S
-from helpers import GRAD_REL, PARAM_NAMES, assert_close_sum, settings
+from helpers import GRAD_REL, PARAM_NAMES, assert_same_sums, settings
 
 pytestmark = pytest.mark.gpu
 H, W, DEV = 48, 64, "cuda"
@@ -64,7 +65,7 @@ def close(a, b, tag):
         if a[k] is None or b[k] is None:
             assert a[k] is None and b[k] is None, (tag, k)
         else:
-            assert_close_sum(a[k], b[k], GRAD_REL, tag + " " + k)
+            assert_same_sums(a[k], b[k], GRAD_REL, tag + " " + k)
 
 
 @pytest.fixture(scope="module")
@@ -107,7 +108,7 @@ def test_only_some_inputs_ask_for_gradients(B, req):
     got = B.grads(lf)
     for k in got:
         if k in req:
-            assert_close_sum(got[k], B.single[1][k], GRAD_REL, "subset " + k)
+            assert_same_sums(got[k], B.single[1][k], GRAD_REL, "subset " + k)
         else:
             assert got[k] is None, k
 
