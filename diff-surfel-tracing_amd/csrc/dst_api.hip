@@ -69,6 +69,7 @@ void dst_destroy(dst_ctx *ctx) {
     if (!ctx) return;
     dst_lbvh_free(ctx);
     if (ctx->bounds) (void)hipFree(ctx->bounds);
+    if (ctx->core_box) (void)hipFree(ctx->core_box);
     if (ctx->bounds_host) (void)hipHostFree(ctx->bounds_host);
     delete ctx;
 }

@@ -114,6 +114,7 @@ struct dst_ctx {
     uint32_t block_order_capacity = 0;
     DstBounds *bounds = nullptr;       // device
     DstBounds *bounds_host = nullptr;  // pinned host copy
+    void *core_box = nullptr;          // device: the box the two-level Morton keys are laid over (lbvh.hip)
     float scene_lo[3] = {0, 0, 0}, scene_hi[3] = {0, 0, 0}, max_abs = 0;
 };
 

@@ -208,11 +208,86 @@ __global__ void k_morton(const float4 *__restrict__ centroids, const DstBounds *
     vals[g] = g;
 }
 
+// The box the two-level keys are laid over: the centroids' bounds, cut down to mean +- 4 sigma per axis, three times
+// over.  One surfel a million scene sizes away (an optimisation step gone wrong) would otherwise shrink the scene to
+// a single cell even of the 2^20 grid; cut off, it lands in a cell at the grid's edge.  A uniform or a normal cloud
+// keeps its bounds (4 sigma lies outside, or takes a few surfels in a hundred thousand to the edge cells).  The sums
+// are integers (coordinates quantised to 16 bits of the current box), so every run cuts at the same place.
+struct CoreBox {
+    float lo[3], hi[3];
+    unsigned long long s0[3], s1[3], s2[3];
+};
+__global__ void k_core_init(CoreBox *core, const DstBounds *__restrict__ bounds) {
+    const int a = threadIdx.x;
+    if (a < 3) {
+        core->lo[a] = ord2f(bounds->lo[a]);
+        core->hi[a] = ord2f(bounds->hi[a]);
+        core->s0[a] = core->s1[a] = core->s2[a] = 0ull;
+    }
+}
+__global__ void k_core_stats(const float4 *__restrict__ centroids, CoreBox *core, uint32_t P) {
+    __shared__ unsigned long long s_sum[kBlock / DST_WAVE][9];
+    float lo[3], sc[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        lo[a] = core->lo[a];
+        const float ext = core->hi[a] - lo[a];
+        sc[a] = (ext > 0.f && ext < INFINITY) ? 65535.0f / ext : 0.f;
+    }
+    unsigned long long acc[9] = {0ull, 0ull, 0ull, 0ull, 0ull, 0ull, 0ull, 0ull, 0ull};
+    for (uint32_t g = blockIdx.x * blockDim.x + threadIdx.x; g < P; g += gridDim.x * blockDim.x) {
+        const float4 c = centroids[g];
+        const float cc[3] = {c.x, c.y, c.z};
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            const float x = (cc[a] - lo[a]) * sc[a];
+            if (x >= 0.f && x <= 65535.f) {   // inside the current box (and not NaN)
+                const unsigned long long q = (unsigned long long)x;
+                acc[a] += 1ull;
+                acc[3 + a] += q;
+                acc[6 + a] += q * q;
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 9; ++k) {
+#pragma unroll
+        for (int o = DST_WAVE / 2; o > 0; o >>= 1) acc[k] += __shfl_xor(acc[k], o);
+    }
+    const int w = threadIdx.x / DST_WAVE;
+    if ((threadIdx.x & (DST_WAVE - 1)) == 0) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) s_sum[w][k] = acc[k];
+    }
+    __syncthreads();
+    if (threadIdx.x < 9) {
+        unsigned long long t = 0ull;
+        for (int k = 0; k < (int)(blockDim.x / DST_WAVE); ++k) t += s_sum[k][threadIdx.x];
+        unsigned long long *dst = threadIdx.x < 3 ? &core->s0[threadIdx.x] : (threadIdx.x < 6 ? &core->s1[threadIdx.x - 3] : &core->s2[threadIdx.x - 6]);
+        if (t != 0ull) atomicAdd(dst, t);
+    }
+}
+__global__ void k_core_cut(CoreBox *core) {
+    const int a = threadIdx.x;
+    if (a >= 3) return;
+    const double n = (double)core->s0[a];
+    if (n > 0.0) {
+        const double mean = (double)core->s1[a] / n;
+        const double var = fmax((double)core->s2[a] / n - mean * mean, 0.0);
+        const double half = 4.0 * sqrt(var) + 1.0;   // and one cell of the 16-bit grid
+        const double q_lo = fmax(mean - half, 0.0), q_hi = fmin(mean + half, 65535.0);
+        const double lo = (double)core->lo[a], ext = (double)core->hi[a] - lo;
+        core->lo[a] = (float)(lo + q_lo / 65535.0 * ext);
+        core->hi[a] = (float)(lo + q_hi / 65535.0 * ext);
+    }
+    core->s0[a] = core->s1[a] = core->s2[a] = 0ull;
+}
+
 // Two-level keys for scenes whose centroids crowd into few cells of the 1024^3 grid (a few surfels far outside an
 // otherwise compact scene stretch the grid over the whole extent): 20 bits per axis, the upper ten interleaved
 // into `hi` (the same cells as k_morton's), the lower ten into `lo`.  Sorted as two stable 32-bit sorts, by `lo`
 // first and then by `hi`, with the same kernels as the one-level keys.
-__global__ void k_morton_fine(const float4 *__restrict__ centroids, const DstBounds *__restrict__ bounds,
+__global__ void k_morton_fine(const float4 *__restrict__ centroids, const CoreBox *__restrict__ core,
                               uint32_t *__restrict__ keys, uint32_t *__restrict__ lo_of, uint32_t *__restrict__ hi_of,
                               uint32_t *__restrict__ vals, uint32_t P) {
     uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
@@ -221,12 +296,12 @@ __global__ void k_morton_fine(const float4 *__restrict__ centroids, const DstBou
     const float cc[3] = {c.x, c.y, c.z};
     float ext = 0.f;
 #pragma unroll
-    for (int a = 0; a < 3; ++a) ext = fmaxf(ext, ord2f(bounds->hi[a]) - ord2f(bounds->lo[a]));
+    for (int a = 0; a < 3; ++a) ext = fmaxf(ext, core->hi[a] - core->lo[a]);
     const float s = (ext > 0.f && ext < INFINITY) ? 1048576.0f / ext : 0.f;
     uint32_t qh[3], ql[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        float x = (cc[a] - ord2f(bounds->lo[a])) * s;
+        float x = (cc[a] - core->lo[a]) * s;   // a surfel outside the box goes to the cell at its edge
         x = fminf(fmaxf(x, 0.f), 1048575.f);  // NaN -> 0
         const uint32_t q = (uint32_t)x;
         qh[a] = q >> 10;
@@ -433,6 +508,22 @@ __global__ void k_tree_depth(const uint32_t *__restrict__ node_parent, const uin
     if (__lane_id() == 0u && depth != 0u) atomicMax(&bounds->max_depth, depth);
 }
 
+// The trace kernels widen every box and every stand-in limit by a multiple of the magnitudes of the numbers that meet
+// in the test: the ray origin's (added per ray) and the quad's own coordinates' (added here, once, to the quad's box
+// and limits).  A scene-wide bound in the quad's place would make the slack of every test grow with the farthest surfel:
+// one of them a thousand scene sizes away and every box of the scene is wider than the surfel inside it.
+constexpr float kBoxPad = 4e-6f;      // box faces, per unit of coordinate magnitude (make_slab has the ray's share)
+constexpr float kPlanePad = 1.5e-4f;  // in-plane slack of the stand-in (make_pre: padw)
+constexpr float kDistPad = 1e-4f;     // slack of the stand-in's distance along the ray (make_pre: tp)
+__device__ __forceinline__ float quad_magnitude(const float (&c)[4][3]) {
+    float m = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int a = 0; a < 3; ++a) m = finite_max(m, fabsf(c[k][a]));
+    return m;
+}
+
 // Leaf record + conservative stand-in of one quad (corners c[0..3] = A,B,C,D, surfel id g) at leaf position i.
 // The plane normals use the fused form the hit test is defined with: cross(x,y).x = fma(x.y, y.z, -(x.z*y.y)), ...
 __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, uint32_t i, DstLeaf *__restrict__ leaves,
@@ -504,7 +595,12 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
     // corner that is `dev` off the mean plane moves a hit by at most 20 dev along the plane; margins of 2.
     float tdev = 40.0f * dev;
     lim0 = lim0 * 1.002f + tdev * mfu;
-    const bool ok = isfinite(mfu) && isfinite(lim0) && isfinite(tdev) && isfinite(rad) && isfinite(cen[0] + cen[1] + cen[2]) &&
+    // the quad's share of the coordinate-dependent slack (the ray's share is added per ray)
+    const float mag = quad_magnitude(c);
+    lim0 += (kPlanePad * mag) * mfu;
+    tdev += kDistPad * mag;
+    const float rad_padded = rad + kPlanePad * mag;
+    const bool ok = isfinite(mfu) && isfinite(lim0) && isfinite(tdev) && isfinite(rad_padded) && isfinite(cen[0] + cen[1] + cen[2]) &&
                     isfinite(nrm[0] + nrm[1] + nrm[2]) && nl > 0.f;
     float pr[16];
 #pragma unroll
@@ -517,7 +613,7 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
     pr[12] = ok ? mfu : INFINITY;
     pr[13] = ok ? lim0 : INFINITY;
     pr[14] = ok ? tdev : INFINITY;
-    pr[15] = ok ? rad : INFINITY;
+    pr[15] = ok ? rad_padded : INFINITY;
     float4 *pdst = reinterpret_cast<float4 *>(&pre[i]);
 #pragma unroll
     for (int k = 0; k < 4; ++k) pdst[k] = make_float4(pr[4 * k], pr[4 * k + 1], pr[4 * k + 2], pr[4 * k + 3]);
@@ -554,10 +650,11 @@ __device__ __forceinline__ void wave_range_boxes(const float (&c)[4][3], bool va
                                                  const RangeBoxes &rb) {
     const uint32_t lane = threadIdx.x % DST_WAVE;
     float box[6], pre[6], suf[6];
+    const float pad = kBoxPad * quad_magnitude(c);
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        box[a] = valid ? fminf(fminf(c[0][a], c[1][a]), fminf(c[2][a], c[3][a])) : INFINITY;
-        box[3 + a] = valid ? fmaxf(fmaxf(c[0][a], c[1][a]), fmaxf(c[2][a], c[3][a])) : -INFINITY;
+        box[a] = valid ? fminf(fminf(c[0][a], c[1][a]), fminf(c[2][a], c[3][a])) - pad : INFINITY;
+        box[3 + a] = valid ? fmaxf(fmaxf(c[0][a], c[1][a]), fmaxf(c[2][a], c[3][a])) + pad : -INFINITY;
     }
 #pragma unroll
     for (int k = 0; k < 6; ++k) pre[k] = suf[k] = box[k];
@@ -714,10 +811,16 @@ __global__ __launch_bounds__(kFitBlock) void k_fit(DstNode *nodes, const uint32_
     if (i >= n) return;
     const DstLeaf &L = leaves[i];
     float box[6];
+    float c[4][3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        box[a] = fminf(fminf(L.A[a], L.B[a]), fminf(L.C[a], L.D[a]));
-        box[3 + a] = fmaxf(fmaxf(L.A[a], L.B[a]), fmaxf(L.C[a], L.D[a]));
+        c[0][a] = L.A[a]; c[1][a] = L.B[a]; c[2][a] = L.C[a]; c[3][a] = L.D[a];
+    }
+    const float pad = kBoxPad * quad_magnitude(c);   // as in wave_range_boxes: the two fits give the same bits
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        box[a] = fminf(fminf(c[0][a], c[1][a]), fminf(c[2][a], c[3][a])) - pad;
+        box[3 + a] = fmaxf(fmaxf(c[0][a], c[1][a]), fmaxf(c[2][a], c[3][a])) + pad;
     }
     uint32_t pp = leaf_parent[i];
     bool local = true;
@@ -857,6 +960,7 @@ int ensure_capacity(dst_ctx *ctx, uint32_t P) {
     ctx->tile_hist_elems = tiles * kRadix + kRadix;
     DST_HIP(ctx, hipMalloc((void **)&ctx->tile_hist, sizeof(uint32_t) * ctx->tile_hist_elems));
     if (!ctx->bounds) DST_HIP(ctx, hipMalloc((void **)&ctx->bounds, sizeof(DstBounds)));
+    if (!ctx->core_box) DST_HIP(ctx, hipMalloc((void **)&ctx->core_box, sizeof(CoreBox)));
     if (!ctx->bounds_host) DST_HIP(ctx, hipHostMalloc((void **)&ctx->bounds_host, sizeof(DstBounds), hipHostMallocDefault));
     ctx->capacity = P;
     return DST_OK;
@@ -975,7 +1079,14 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
         if (ctx->fine_keys) {
             // second-level keys in original order wait in two buffers that are idle until the hierarchy is made
             uint32_t *lo_of = ctx->node_parent, *hi_of = ctx->flags;
-            hipLaunchKernelGGL(k_morton_fine, grid_for(n), dim3(kBlock), 0, stream, centroids, ctx->bounds, ctx->keys[0],
+            CoreBox *core = reinterpret_cast<CoreBox *>(ctx->core_box);
+            hipLaunchKernelGGL(k_core_init, dim3(1), dim3(64), 0, stream, core, ctx->bounds);
+            for (int pass = 0; pass < 3; ++pass) {
+                hipLaunchKernelGGL(k_core_stats, dim3(std::min<uint32_t>(grid_for(n).x, 256u)), dim3(kBlock), 0, stream,
+                                   centroids, core, n);
+                hipLaunchKernelGGL(k_core_cut, dim3(1), dim3(64), 0, stream, core);
+            }
+            hipLaunchKernelGGL(k_morton_fine, grid_for(n), dim3(kBlock), 0, stream, centroids, core, ctx->keys[0],
                                lo_of, hi_of, ctx->vals[0], n);
             dst_sort_pairs(ctx->keys, ctx->vals, ctx->tile_hist, n, stream);
             hipLaunchKernelGGL(k_gather_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->keys[0], hi_of, ctx->vals[0], n);

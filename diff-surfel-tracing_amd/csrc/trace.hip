@@ -237,10 +237,11 @@ __device__ __forceinline__ RaySlab make_slab(F3 o, F3 d, float max_abs) {
     s.ny = -o.y * s.iy;
     s.nz = -o.z * s.iz;
     // The quad test works in origin-relative fp32 coordinates, so it can accept a ray that passes
-    // a few ulps of (|o| + |vertex|) outside the quad; boxes are widened by well above that.
+    // a few ulps of (|o| + |vertex|) outside the quad; boxes are widened by well above that: by 4e-6 |o| here,
+    // and by 4e-6 of the quad's own largest coordinate where the boxes are made (lbvh.hip, kBoxPad).
     float oa = __builtin_fmaxf(__builtin_fabsf(o.x), __builtin_fmaxf(__builtin_fabsf(o.y), __builtin_fabsf(o.z)));
     s.max_abs = max_abs;
-    float pad = 4e-6f * (oa + max_abs);
+    float pad = 4e-6f * oa;
     s.wx = pad * __builtin_fabsf(s.ix);
     s.wy = pad * __builtin_fabsf(s.iy);
     s.wz = pad * __builtin_fabsf(s.iz);
@@ -322,7 +323,7 @@ struct WaveStats { unsigned long long nodes, leaves, t_trav, t_comp, chunks, lea
 #endif
 
 // Per-lane constants of the conservative stand-in for the quad test (DstLeafPre).  With S = |o|_max + the largest
-// vertex coordinate: the stand-in's distance along the ray is off by at most about 3.4e-5 S/|d| + 1e-5 |t| when
+// coordinate of the quad: the stand-in's distance along the ray is off by at most about 3.4e-5 S/|d| + 1e-5 |t| when
 // |n.d| >= 0.05 |d| (flatter rays skip the stand-in), its hit point by 7e-5 S; the margins below are twice that.
 struct RayPre {
     float padw;     // in-plane slack, world units
@@ -333,7 +334,7 @@ struct RayPre {
 __device__ __forceinline__ RayPre make_pre(F3 o, F3 d, float max_abs) {
     RayPre r;
     const float oa = __builtin_fmaxf(__builtin_fabsf(o.x), __builtin_fmaxf(__builtin_fabsf(o.y), __builtin_fabsf(o.z)));
-    const float S = oa + max_abs;
+    const float S = oa;   // the ray's share; the quad's own coordinates are in its limits already (lbvh.hip, write_leaf)
     const float dl = __builtin_sqrtf(d.x * d.x + d.y * d.y + d.z * d.z);
     r.inv_dl = 1.0f / dl;
     r.padw = 1.5e-4f * S;

@@ -43,8 +43,17 @@ def check_tree(info, nodes, leaves, npar, lpar, keys, vertices):
     A, B, C, D = (leaves[c].astype(np.float64) for c in "ABCD")
     np.testing.assert_allclose(leaves["n0"], np.cross(B - A, C - A), rtol=1e-4, atol=1e-7)   # plane normals
     np.testing.assert_allclose(leaves["n1"], np.cross(C - B, D - B), rtol=1e-4, atol=1e-7)
-    llo = np.minimum.reduce([leaves[c] for c in "ABCD"])
-    lhi = np.maximum.reduce([leaves[c] for c in "ABCD"])
+    # a leaf's box: its corners, widened by 4e-6 of the quad's largest coordinate (the quad's share of the slack the
+    # box tests need; computed in fp32 like the kernel does)
+    with np.errstate(invalid="ignore"):
+        mag = np.zeros(n, np.float32)
+        for c in "ABCD":
+            a = np.abs(leaves[c])
+            mag = np.maximum(mag, np.where(np.isfinite(a), a, np.float32(0)).max(1))
+    pad = (np.float32(4e-6) * mag)[:, None]
+    llo = np.minimum.reduce([leaves[c] for c in "ABCD"]) - pad
+    lhi = np.maximum.reduce([leaves[c] for c in "ABCD"]) + pad
+    assert llo.dtype == np.float32 and lhi.dtype == np.float32
     # walk from the root: every node and leaf reached once, parents consistent, boxes = exact union of content
     seen_nodes, seen_leaves = np.zeros(n - 1, bool), np.zeros(n, bool)
     box_lo, box_hi = {}, {}
@@ -152,11 +161,13 @@ def test_surfels_far_outside_a_compact_scene_switch_the_builds_to_two_level_keys
 
 def test_two_level_keys_are_given_up_when_the_hierarchy_gets_too_deep():
     """Sixty surfels that each peel one bit off the 60-bit key (one per axis and scale, down to a millionth of the
-    extent) in front of 4096 surfels at one point: with two-level keys the deepest leaf lies 72 nodes down, more than
-    the walks' stacks are sized for.  The build measures that and returns to one-level keys for good."""
+    extent) in front of 16384 surfels at one point, and a uniform cloud that keeps the box of the keys at full
+    size: with two-level keys the deepest leaf lies 74 nodes down, more than the walks' stacks are sized for.  The
+    build measures that and returns to one-level keys for good."""
     import diff_surfel_tracing as dst
     own = dst.SurfelTracer()
-    pts = [[0.0, 0.0, 0.0]] * 4096
+    pts = [[0.0, 0.0, 0.0]] * 16384
+    pts += (torch.rand(4096, 3, generator=torch.Generator().manual_seed(3)) * 1.2).tolist()
     for k in range(20):
         for a in range(3):
             p = [0.0, 0.0, 0.0]
@@ -171,7 +182,7 @@ def test_two_level_keys_are_given_up_when_the_hierarchy_gets_too_deep():
     info, *arrs = download(own)
     assert info.key_levels == 1 and info.builds == 1
     depth = check_tree(info, *arrs, sc["vertices"].numpy())
-    assert 40 <= depth < 62        # thirty peeled bits, then the 4096 + 30 surfels of the last cell
+    assert 40 <= depth < 62        # thirty peeled bits, then the 16384 + 30 surfels of the last cell
     # the refusal holds: a scene that asks for two levels again is built with one
     far = _with_far_surfels(S.scene_cube(P=3000, seed=8), 2000.0)
     own.build_acceleration_structure(far["vertices"].cuda(), far["faces"].cuda(), True)
