@@ -68,6 +68,8 @@ struct DstBounds {          // device-resident reduction targets, order-preservi
     uint32_t bad_topology;  // set by the quad set-up kernel
     uint32_t equal_keys;    // neighbours in Morton order with equal keys, counted while the hierarchy is made
     uint32_t max_depth;     // nodes above the deepest leaf (builds with two-level keys only)
+    uint32_t scale;         // raw bits of a float: size of the scene's bulk (set by a build, kept by refits); what ray
+                            // origins are compared with (packets, ray keys) - not a bound on anything
 };
 
 // Device-side view of the acceleration structure handed to the trace kernels.

@@ -283,6 +283,18 @@ __global__ void k_core_cut(CoreBox *core) {
     core->s0[a] = core->s1[a] = core->s2[a] = 0ull;
 }
 
+// Size of the scene's bulk: the largest coordinate of the keys' box (two-level keys: the cut box), else of any vertex.
+__global__ void k_scene_scale(DstBounds *bounds, const CoreBox *core) {
+    if (threadIdx.x != 0) return;
+    float m = __uint_as_float(bounds->max_abs);
+    if (core != nullptr) {
+        float c = 0.f;
+        for (int a = 0; a < 3; ++a) c = finite_max(c, fmaxf(fabsf(core->lo[a]), fabsf(core->hi[a])));
+        if (c > 0.f) m = fminf(m, c);
+    }
+    bounds->scale = __float_as_uint(m);
+}
+
 // Two-level keys for scenes whose centroids crowd into few cells of the 1024^3 grid (a few surfels far outside an
 // otherwise compact scene stretch the grid over the whole extent): 20 bits per axis, the upper ten interleaved
 // into `hi` (the same cells as k_morton's), the lower ten into `lo`.  Sorted as two stable 32-bit sorts, by `lo`
@@ -1086,6 +1098,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
                                    centroids, core, n);
                 hipLaunchKernelGGL(k_core_cut, dim3(1), dim3(64), 0, stream, core);
             }
+            hipLaunchKernelGGL(k_scene_scale, dim3(1), dim3(64), 0, stream, ctx->bounds, core);
             hipLaunchKernelGGL(k_morton_fine, grid_for(n), dim3(kBlock), 0, stream, centroids, core, ctx->keys[0],
                                lo_of, hi_of, ctx->vals[0], n);
             dst_sort_pairs(ctx->keys, ctx->vals, ctx->tile_hist, n, stream);
@@ -1093,6 +1106,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
             dst_sort_pairs(ctx->keys, ctx->vals, ctx->tile_hist, n, stream);   // stable: equal cells stay in `lo` order
             hipLaunchKernelGGL(k_gather_u32, grid_for(n), dim3(kBlock), 0, stream, ctx->keys[1], lo_of, ctx->vals[0], n);
         } else {
+            hipLaunchKernelGGL(k_scene_scale, dim3(1), dim3(64), 0, stream, ctx->bounds, (const CoreBox *)nullptr);
             hipLaunchKernelGGL(k_morton, grid_for(n), dim3(kBlock), 0, stream, centroids, ctx->bounds, ctx->keys[0],
                                ctx->vals[0], n);
             dst_sort_pairs(ctx->keys, ctx->vals, ctx->tile_hist, n, stream);   // the sorted pairs end in buffer 0

@@ -1859,7 +1859,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     const size_t pos = inside ? ((size_t)py * p.W + px) : 0;
     // (forward: ray lists always run the MIXED kernels, so the image kernels need not look at the order)
     const size_t r = ((MIXED || BWD) && ray_order != nullptr && inside) ? (size_t)ray_order[pos] : pos;
-    const float max_abs = __uint_as_float(acc.bounds->max_abs);
+    const float max_abs = __uint_as_float(acc.bounds->scale);   // the size origins are compared with (rays_run_together)
     const int MID = 14 + p.aux, AUXO = 11, RGBO = 11 + p.aux;
     const int slots = p.mtd_alloc + 1, mtd = p.max_trace_depth;
     float *mid = p.mid_val + (size_t)slots * MID * r;
@@ -2125,7 +2125,7 @@ __global__ void k_ray_keys(const float *__restrict__ ray_o, const float *__restr
                            uint32_t *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t n) {
     const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= n) return;
-    const float ext = __uint_as_float(bounds->max_abs);
+    const float ext = __uint_as_float(bounds->scale);
     const float inv = ext > 0.f ? 16.0f / ext : 0.f;
     uint32_t cell = 0u, dir = 0u;
     float d[3], l1 = 0.f;
