@@ -2,7 +2,8 @@
 surfel count from 3 to 40 000, surfel size x0.3 to x10, image from 1x1 to 71x71 (or the same rays as a list, or
 unrelated rays), aux channels, SH degree, depth 0 to 2 with thresholds, background, `start_from_first`; a degenerate
 trait (all surfels at one point, zero scales, a scene 3 km from the origin, 25:1 quads, a scene of 0.1 mm or 30 km,
-opacities of exactly 0 and 1, a flat scene seen head-on and edge-on, NaN and infinite parameters); and the mode of the
+opacities of exactly 0 and 1, a flat scene seen head-on and edge-on, NaN and infinite parameters, a few surfels a
+thousand to a million scene sizes away); and the mode of the
 call (plain, deterministic, without a hit record, without gradient rows, after a refit, after a refit from the
 surfel parameters).  The cases are small; their value is in the combinations no hand-written test makes."""
 import os
@@ -16,7 +17,8 @@ from test_gpu_parity import _with_scales, check_case
 
 pytestmark = pytest.mark.gpu
 
-TRAITS = ("none", "none", "samepoint", "zero_scale", "far_away", "elongated", "tiny", "huge", "opacity", "flat_z", "nonfinite")
+TRAITS = ("none", "none", "samepoint", "zero_scale", "far_away", "elongated", "tiny", "huge", "opacity", "flat_z", "nonfinite",
+          "outliers")
 MODES = ("plain", "plain", "det", "norec", "norows", "refit", "refit_surfels")
 
 
@@ -73,6 +75,11 @@ def _apply_trait(sc, trait, gen):
     elif trait == "flat_z":
         sc["means3D"][:, 2] = 0.0
         sc["rotations"] = torch.tensor([1.0, 0.0, 0.0, 0.0]).repeat(P, 1).contiguous()
+    elif trait == "outliers":
+        k = max(1, P // 500)
+        dirs = torch.nn.functional.normalize(torch.randn(k, 3, generator=gen), dim=-1)
+        far = 10.0 ** (3.0 + 3.0 * torch.rand(k, 1, generator=gen))       # 1e3 to 1e6 scene sizes away
+        sc["means3D"][:k] = dirs * far * float(sc["means3D"].abs().max())
     elif trait == "nonfinite":
         r = torch.rand(P, generator=gen)
         sc["means3D"][r < 0.02, 0] = float("nan")
@@ -146,6 +153,10 @@ def test_random_configuration(oracle, tracer, case):
     if depth > 0:
         kw.update(max_trace_depth=depth, specular_threshold=float(rng.choice([0.0, 0.1, 0.4])))
     grads = True
+    if trait == "outliers":
+        # its builds go over to two-level keys for good: a context of its own, the session's keeps its one-level keys
+        import diff_surfel_tracing as dst
+        tracer = dst.SurfelTracer()
     ctx = tracer.optix_context
     saved = (ctx.record_max_bytes, ctx.gradient_rows)
     try:
