@@ -5,6 +5,7 @@
 """
 import ctypes as C
 import os
+import warnings
 
 import torch
 
@@ -177,11 +178,14 @@ class OptiXStateWrapper:
     change.  `pkg_dir` was where the reference looked for its PTX files and is ignored.
 
     Also owns the hit-record buffers of the autograd path: a small pool that forward calls draw from and
-    backward calls return to (no allocation per call once warm), bounded by `record_max_bytes` per record; a
-    record that would be larger, or whose allocation fails, is simply not made and the backward pass walks the
-    BVH again."""
+    backward calls return to (no allocation per call once warm), bounded by `record_max_bytes` per record and
+    `record_pool_max_bytes` for the free storages together; a record that would be larger, or whose allocation
+    fails, is not made and the backward pass walks the BVH again (`records_skipped` counts those calls, the first
+    one warns)."""
 
     RECORD_POOL_SIZE = 4
+    RECORD_FIRST_BLOCKS = 5.0   # blocks per wave and bounce before a forward trace has said what it needs
+    RECORD_HEADROOM = 1.08      # a record is sized this much above the largest request seen so far
 
     def __init__(self, pkg_dir=None):
         lib = load_library()
@@ -192,13 +196,16 @@ class OptiXStateWrapper:
             raise RuntimeError("dst_create failed: no usable HIP device")
         self.device = torch.cuda.current_device()
         self.num_surfels = 0
-        self.record_blocks_per_wave = 6.0   # sizing estimate for hit records, raised when a record overflows
+        self.record_blocks_per_wave = None  # sizing estimate for hit records: largest request seen, with headroom
         self.record_max_bytes = 8 << 30     # no record larger than this is made (backward then re-traces)
+        self.record_pool_max_bytes = 16 << 30   # free storages kept for reuse, all together
+        self.records_skipped = 0            # forward calls that made no record because of the two limits above
         self.record_wanted = True           # set by the autograd wrapper for the call that follows
         self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
         self.gradient_rows = True           # backward sums per-surfel gradients in one row per surfel first (faster)
         self.distortion = False             # True: the dist output carries the 2DGS depth distortion (else zeros)
         self._record_pool = []              # free storages (int64 tensors)
+        self._record_events = {}            # id(storage) -> event recorded when the storage came back
         self._record_fixed = False          # True: only caller-provided storage is used, nothing is allocated
         self._record_watch = []             # records whose request count has not been read yet
 
@@ -221,16 +228,27 @@ class OptiXStateWrapper:
             if asked is None:
                 still.append(rec)
             else:
-                self.record_blocks_per_wave = max(self.record_blocks_per_wave, 1.25 * asked / rec.n_waves)
+                self.record_blocks_per_wave = max(self.record_blocks_per_wave or 0.0,
+                                                  self.RECORD_HEADROOM * asked / rec.n_waves)
         self._record_watch = still[-8:]
 
-    def acquire_record(self, H, W, mtd_alloc, device):
+    def acquire_record(self, H, W, mtd_alloc, device, max_trace_depth=None):
+        """A record for an (H,W) grid traced with `mtd_alloc` mid_val slots - 1, or None.  Sized from what earlier
+        forward traces asked for (with a little headroom); before any has finished, for RECORD_FIRST_BLOCKS blocks
+        per wave and bounce actually traced (`max_trace_depth` + 1; `mtd_alloc` + 1 if that is not given): every bounce
+        of a path opens at least one block per wave, so a multi-bounce run can replay from its first step."""
         self.update_record_estimate()
-        # every bounce of a path opens at least one block per wave: before anything has been learned from a finished
-        # forward trace, a multi-bounce record is sized for that many more
-        per_wave = max(self.record_blocks_per_wave, 4.0 * (mtd_alloc + 1))
+        per_wave = self.record_blocks_per_wave
+        if per_wave is None:
+            bounces = (mtd_alloc if max_trace_depth is None else max_trace_depth) + 1
+            per_wave = self.RECORD_FIRST_BLOCKS * bounces
         words = HitRecord.layout(H, W, mtd_alloc, per_wave)[0]
         if 8 * words > self.record_max_bytes:
+            self.records_skipped += 1
+            if self.records_skipped == 1:
+                warnings.warn("diff_surfel_tracing: a hit record for this %dx%d trace would take %.1f GiB (limit "
+                              "record_max_bytes = %.1f GiB); backward passes walk the BVH again instead of replaying"
+                              % (H, W, 8 * words / 2 ** 30, self.record_max_bytes / 2 ** 30))
             return None
         device = torch.device(device)
         if device.index is None:
@@ -240,24 +258,39 @@ class OptiXStateWrapper:
         if fit:
             storage = min(fit, key=lambda t: t.numel())
             self._record_pool = [t for t in self._record_pool if t is not storage]
+            # the backward trace that last read this storage may still be running on another stream
+            done = self._record_events.pop(id(storage), None)
+            if done is not None:
+                torch.cuda.current_stream().wait_event(done)
         elif self._record_fixed:
             return None
         else:
             try:
-                storage = torch.empty(words + words // 8, dtype=torch.int64, device=device)
+                storage = torch.empty(words, dtype=torch.int64, device=device)
             except torch.OutOfMemoryError:
+                self.records_skipped += 1
                 return None
         return HitRecord(H, W, mtd_alloc, per_wave, device, storage=storage)
 
     def release_record(self, rec):
+        """Back to the pool.  The storage's last reader (a backward trace just enqueued on the current stream) is
+        marked with an event that the next user waits for, whatever stream that user runs on."""
         if rec is None or rec.words is None:
             return
+        if rec.words.is_cuda:
+            done = torch.cuda.Event()
+            done.record()
+            self._record_events[id(rec.words)] = done
         self._record_pool.append(rec.words)
         rec.words = None
-        if not self._record_fixed and len(self._record_pool) > self.RECORD_POOL_SIZE:
-            # by identity: list.remove() would compare tensors element-wise
+        if self._record_fixed:
+            return
+        # by identity: list.remove() would compare tensors element-wise
+        while len(self._record_pool) > 1 and (len(self._record_pool) > self.RECORD_POOL_SIZE or
+                                              8 * sum(t.numel() for t in self._record_pool) > self.record_pool_max_bytes):
             smallest = min(self._record_pool, key=lambda t: t.numel())
             self._record_pool = [t for t in self._record_pool if t is not smallest]
+            self._record_events.pop(id(smallest), None)
 
     def accel_info(self):
         info = DstAccelInfo()

@@ -68,7 +68,8 @@ class _TraceSurfels(torch.autograd.Function):
         record = None
         if optix_context.record_wanted and any(ctx.needs_input_grad) and ray_o.dim() == 3 and ray_o.numel() > 0:
             record = optix_context.acquire_record(ray_o.size(0), ray_o.size(1),
-                                                  max(_C.DEFAULT_MAX_TRACE_DEPTH, s.max_trace_depth), ray_o.device)
+                                                  max(_C.DEFAULT_MAX_TRACE_DEPTH, s.max_trace_depth), ray_o.device,
+                                                  max_trace_depth=s.max_trace_depth)
         try:
             out_rgb, out_dpt, out_acc, out_norm, out_dist, out_aux, mid_val, a_weights = _guarded(
                 lambda *a: _C.trace_surfels(*a, hit_record=record), args, s.debug, "snapshot_fw.dump", "forward")

@@ -84,7 +84,38 @@ def _report(name, a, b, err, tol, bad, noisy):
                                                        err[k], tol[k]))
 
 
-def assert_close_sum(a, b, rel, name, noise=None, max_noisy=0.02):
+# What the noise allowance was actually used for, per compared tensor: (name, elements, needing the noise term,
+# whose noise term alone exceeds LOUD_NOISE of the value).  conftest prints it at the end of a run.
+NOISE_LOG = []
+LOUD_NOISE = 0.3
+
+
+def _same_nonfinite(a, b, name):
+    """NaN / +inf / -inf must sit in the same places on both sides; returns the mask of finite elements."""
+    fa, fb = np.isfinite(a), np.isfinite(b)
+    assert np.array_equal(fa, fb), "%s: %d elements are finite on one side only" % (name, int((fa != fb).sum()))
+    if not fa.all():
+        bad = ~fa
+        same = (np.isnan(a[bad]) & np.isnan(b[bad])) | (a[bad] == b[bad])
+        assert same.all(), "%s: %d non-finite elements differ in kind (nan, +inf, -inf)" % (name, int((~same).sum()))
+    return fa
+
+
+def _noise_rules(name, err, base, extra, ref_abs, max_noisy, finite):
+    """The two rules that keep the rounding-noise allowance from hiding a defect: few elements may need it at all,
+    and only a handful may carry an allowance that is itself a sizeable part of the value."""
+    noisy = (err > base) & finite
+    loud = np.zeros_like(noisy) if np.isscalar(extra) else ((extra > LOUD_NOISE * ref_abs) & (ref_abs > base) & finite)
+    NOISE_LOG.append((name, int(noisy.size), int(noisy.sum()), int(loud.sum())))
+    assert noisy.sum() <= max(max_noisy * noisy.size, MIN_NOISY), (
+        "%s: %d of %d elements (%.3g) pass only through the noise allowance" % (name, noisy.sum(), noisy.size, noisy.mean()))
+    assert loud.sum() <= max(MAX_LOUD * loud.size, MIN_NOISY), (
+        "%s: the noise allowance alone exceeds %.0f %% of the value on %d of %d elements" % (
+            name, 100 * LOUD_NOISE, loud.sum(), loud.size))
+    return noisy
+
+
+def assert_close_sum(a, b, rel, name, noise=None, max_noisy=None):
     """Sums accumulated in a different order on the two sides (atomics on the GPU, double accumulators in the
     oracle): ELEMENT-WISE |a - b| <= rel * |b| + floor + NOISE_FACTOR * noise.
     floor: rel/20 of the root-mean-square of the channel's nonzero entries (a sum that cancels keeps the rounding
@@ -94,25 +125,27 @@ def assert_close_sum(a, b, rel, name, noise=None, max_noisy=0.02):
     geometric gradients, its first-order sensitivity to one unit of rounding in the plane-hit chain (a grazing
     hit at 50 m divides a difference of two 50 m vectors by n.d twice: one ulp in t = n.(v1-o)/n.d moves such an
     element by tens of per cent).  No fp32 implementation, the reference's included, is closer to another than that.
-    At most `max_noisy` of the elements (or MIN_NOISY of them, for a tensor of a few dozen) may owe their pass to the
-    noise term."""
+    At most MAX_NOISY of the elements (or MIN_NOISY of them, for a small tensor) may owe their pass to the noise
+    term, and at most MAX_LOUD of them may carry a noise term above LOUD_NOISE of the value itself.  NaN and
+    infinities must sit at the same places on both sides."""
+    max_noisy = MAX_NOISY if max_noisy is None else max_noisy
     assert a.shape == b.shape, (name, a.shape, b.shape)
     a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
     flat_b = b64.reshape(-1, b64.shape[-1]) if b64.ndim > 1 else b64.reshape(-1, 1)
     flat_a = a64.reshape(flat_b.shape)
-    assert np.isfinite(flat_a).all() == np.isfinite(flat_b).all(), name
-    live = flat_b != 0
-    rms = np.sqrt((flat_b ** 2).sum(0) / np.maximum(live.sum(0), 1))
-    base = rel * np.abs(flat_b) + rel / 20 * rms[None, :]
-    extra = 0.0 if noise is None else NOISE_FACTOR * np.asarray(noise, np.float64).reshape(flat_b.shape)
-    err = np.abs(flat_a - flat_b)
+    finite = _same_nonfinite(flat_a, flat_b, name)
+    fb = np.where(finite, flat_b, 0.0)
+    live = fb != 0
+    rms = np.sqrt((fb ** 2).sum(0) / np.maximum(live.sum(0), 1))
+    base = rel * np.abs(fb) + rel / 20 * rms[None, :]
+    extra = 0.0 if noise is None else NOISE_FACTOR * np.nan_to_num(np.asarray(noise, np.float64).reshape(flat_b.shape),
+                                                                    nan=0.0, posinf=0.0, neginf=0.0)
+    err = np.where(finite, np.abs(np.where(finite, flat_a, 0.0) - fb), 0.0)
     tol = base + extra
     bad = err > tol
-    noisy = (err > base)
     if bad.any():
-        raise AssertionError(_report(name, flat_a, flat_b, err, tol, bad, noisy))
-    assert noisy.sum() <= max(max_noisy * noisy.size, MIN_NOISY), (
-        "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean()))
+        raise AssertionError(_report(name, flat_a, flat_b, err, tol, bad, err > base))
+    _noise_rules(name, err, base, extra, np.abs(fb), max_noisy, finite)
 
 
 def assert_same_sums(a, b, rel, name):
@@ -129,21 +162,25 @@ def assert_same_sums(a, b, rel, name):
         name, int(bad.sum()), bad.size, float((err / np.maximum(tol, 1e-300)).max()))
 
 
-def assert_close_rays(a, b, rel, name, noise=None, max_noisy=0.02):
+def assert_close_rays(a, b, rel, name, noise=None, max_noisy=None):
     """Per-ray gradients are plain stores (no atomics): element-wise |a - b| <= rel * |b| + rel/10 * (largest
-    component of that ray's gradient) + NOISE_FACTOR * noise (see assert_close_sum)."""
+    component of that ray's gradient) + NOISE_FACTOR * noise (see assert_close_sum, also for the rules on how many
+    elements may lean on the noise term and on non-finite values)."""
+    max_noisy = MAX_NOISY if max_noisy is None else max_noisy
     assert a.shape == b.shape, (name, a.shape, b.shape)
     a64, b64 = np.asarray(a, np.float64), np.asarray(b, np.float64)
-    row = np.abs(b64).max(-1, keepdims=True)
-    base = rel * np.abs(b64) + rel / 10 * row + 1e-30
-    extra = 0.0 if noise is None else NOISE_FACTOR * np.asarray(noise, np.float64)
-    err, tol = np.abs(a64 - b64), base + extra
+    finite = _same_nonfinite(a64, b64, name)
+    fb = np.where(finite, b64, 0.0)
+    row = np.abs(fb).max(-1, keepdims=True)
+    base = rel * np.abs(fb) + rel / 10 * row + 1e-30
+    extra = 0.0 if noise is None else NOISE_FACTOR * np.nan_to_num(np.asarray(noise, np.float64), nan=0.0, posinf=0.0,
+                                                                    neginf=0.0)
+    err = np.where(finite, np.abs(np.where(finite, a64, 0.0) - fb), 0.0)
+    tol = base + extra
     bad = err > tol
-    noisy = err > base
     if bad.any():
-        raise AssertionError(_report(name, a64, b64, err, tol, bad, noisy))
-    assert noisy.sum() <= max(max_noisy * noisy.size, MIN_NOISY), (
-        "%s: %.3g of the elements pass only through the noise allowance" % (name, noisy.mean()))
+        raise AssertionError(_report(name, a64, b64, err, tol, bad, err > base))
+    _noise_rules(name, err, base, extra, np.abs(fb), max_noisy, finite)
 
 
 def assert_gradients(got, ref32, ref64, rel, tag=""):
@@ -167,7 +204,10 @@ def assert_gradients(got, ref32, ref64, rel, tag=""):
         (assert_close_rays if k in ("ray_o", "ray_d") else assert_close_sum)(got[k], want, rel, tag + k, noise=noise)
 
 
-MIN_NOISY = 4     # a share of 2 % is no measure on a tensor of 80 elements
+MAX_NOISY = 2e-3  # share of a tensor's elements that may need the noise term (observed: 1.1e-3 on the sphere of config 2,
+                  # whose silhouette is all grazing hits; at most 7e-5 on configs 3, 4 and 5 at full size)
+MAX_LOUD = 2e-2   # share whose noise term alone may exceed LOUD_NOISE of the value (observed: 9e-3 on config 2, 9e-4 on 3)
+MIN_NOISY = 4     # a share is no measure on a tensor of 80 elements
 GRAD_REL = 1e-3   # north star: gradients within 1e-3 relative
 OUT_ABS = 1e-4    # north star: rendered outputs within 1e-4 absolute (we get bit equality)
 

@@ -149,7 +149,7 @@ class _FakeContext:
         self.acquired = 0
         self.released = 0
 
-    def acquire_record(self, H, W, mtd_alloc, device):
+    def acquire_record(self, H, W, mtd_alloc, device, max_trace_depth=None):
         self.acquired += 1
         return None   # "too large": the backward pass would walk the BVH again
 
@@ -199,7 +199,8 @@ def test_record_pool_takes_back_records_of_any_size():
             self.words = torch.zeros(n, dtype=torch.int64)
 
     pool = _C.OptiXStateWrapper.__new__(_C.OptiXStateWrapper)   # no device: only the pool's bookkeeping is used
-    pool._record_pool, pool._record_fixed = [], False
+    pool._record_pool, pool._record_fixed, pool._record_events = [], False, {}
+    pool.record_pool_max_bytes = 1 << 40
     sizes = [7, 3, 9, 3, 5, 11, 2, 9]
     recs = [_Rec(n) for n in sizes]
     for r in recs:
@@ -210,3 +211,10 @@ def test_record_pool_takes_back_records_of_any_size():
     pool.release_record(recs[0])    # a record already handed back is ignored
     pool.release_record(None)
     assert len(pool._record_pool) == _C.OptiXStateWrapper.RECORD_POOL_SIZE
+    # the free storages are also bounded in bytes, whatever their number: the smallest go first, one always stays
+    pool.record_pool_max_bytes = 8 * 21
+    pool.release_record(_Rec(1))
+    assert sorted(t.numel() for t in pool._record_pool) == [9, 11]
+    pool.record_pool_max_bytes = 8
+    pool.release_record(_Rec(4))
+    assert [t.numel() for t in pool._record_pool] == [11]

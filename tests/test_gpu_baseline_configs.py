@@ -58,7 +58,7 @@ def test_config2_sphere_100k_800x800_build_once_then_refit(oracle, tracer):
 
 
 def test_config5_lidar_refit_loop_20_frames(oracle, tracer):
-    """BASELINE config 5 at a tenth of its size (200k surfels, 64 beams x 256 azimuths as a (1,N,3) ray list, 4 aux
+    """BASELINE config 5's sequence of 20 refits at a tenth of its size (200k surfels, 64 beams x 256 azimuths as a (1,N,3) ray list, 4 aux
     channels): 20 frames of perturb 10 % of the means -> refit -> forward + backward, each frame against the oracle
     (which builds its own BVH from the frame's quads)."""
     sc = S.scene_lidar(P=200000, seed=0, aux=4)
@@ -72,6 +72,25 @@ def test_config5_lidar_refit_loop_20_frames(oracle, tracer):
         compare_all(oracle, tracer, frame_sc, o, d, ug, rebuild=False, tag="config5 frame %d " % frame)
     info = tracer.optix_context.accel_info()
     assert info.builds == builds and info.refits >= 20
+
+
+def test_config5_lidar_full_size_perturb_and_refit(oracle, tracer):
+    """BASELINE config 5 at its real size: 2,000,000 surfels, 64 beams x 2048 azimuths as a (1,131072,3) ray list,
+    4 aux channels; build, then three frames of perturb 10 % of the means -> refit -> forward + backward, each frame
+    against the oracle (about 9 composited hits per ray here; the tenth-size loop above has less than one)."""
+    sc = S.scene_lidar(P=2000000, seed=0, aux=4)
+    o, d = S.rays_lidar()
+    assert o.shape == (1, 131072, 3)
+    ug = upstream(o.shape[0], o.shape[1], 4)
+    ref, _ = compare_all(oracle, tracer, sc, o, d, ug, rebuild=True, tag="config5 full, built ")
+    assert ref["n_con"].mean() > 5
+    builds = tracer.optix_context.accel_info().builds
+    frame_sc = sc
+    for frame in range(1, 4):
+        frame_sc = S.perturb_means(frame_sc, frame)
+        compare_all(oracle, tracer, frame_sc, o, d, ug, rebuild=False, tag="config5 full, frame %d " % frame)
+    info = tracer.optix_context.accel_info()
+    assert info.builds == builds and info.refits >= 3 and info.n_surfels == 2000000
 
 
 def test_config4_room_500k_720p_depth2_forward_and_backward(oracle, tracer):

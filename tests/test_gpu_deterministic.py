@@ -55,7 +55,7 @@ def test_two_runs_are_bit_identical_and_match_the_oracle(oracle, tracer, case):
     finally:
         tracer.deterministic = False
         ctx.record_max_bytes = saved_cap
-        ctx.record_blocks_per_wave = max(saved, 6.0)
+        ctx.record_blocks_per_wave = max(saved or 0.0, 6.0)
     out, g = runs[0]
     s = oracle_scene(oracle, sc, o, d, **kw)
     ref = oracle.forward(s, oracle.HITS_BVH_LEXI)

@@ -326,7 +326,7 @@ def test_backward_replays_the_forward_hit_record_or_retraces(oracle, tracer):
         ctx.update_record_estimate()
         assert ctx.record_blocks_per_wave > 1.0   # learnt from the overflow, without the backward call waiting for it
     finally:
-        ctx.record_blocks_per_wave = max(saved, ctx.record_blocks_per_wave)
+        ctx.record_blocks_per_wave = max(saved or 0.0, ctx.record_blocks_per_wave)
 
 
 @pytest.mark.parametrize("case", ["cube_sh3", "room_aux8_depth2"])
