@@ -948,7 +948,9 @@ int ensure_capacity(dst_ctx *ctx, uint32_t P) {
     const size_t tiles = (n + kTile - 1) / kTile;
     DST_HIP(ctx, hipMalloc((void **)&ctx->nodes, sizeof(DstNode) * std::max<size_t>(n - 1, 1)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->wide, sizeof(DstWideNode) * std::max<size_t>(n - 1, 1)));
-    DST_HIP(ctx, hipMalloc((void **)&ctx->leaves, sizeof(DstLeaf) * n));
+    // (two spare records: the per-lane walk reads a leaf group as eight or ten 16-byte words whatever its size)
+    DST_HIP(ctx, hipMalloc((void **)&ctx->leaves, sizeof(DstLeaf) * (n + 2)));
+    DST_HIP(ctx, hipMemset(ctx->leaves + n, 0, 2 * sizeof(DstLeaf)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->pre, sizeof(DstLeafPre) * (n + 1)));   // the trace kernels fetch them in pairs
     DST_HIP(ctx, hipMemset(ctx->pre + n, 0, sizeof(DstLeafPre)));
     DST_HIP(ctx, hipMalloc((void **)&ctx->node_parent, sizeof(uint32_t) * n));

@@ -169,6 +169,7 @@ __device__ __forceinline__ void load_uniform(const void *p, uint32_t (&out)[N]) 
 // A whole traversal node in one trip: the six face arrays picked by byte offset (scalar-register offsets, so no
 // address arithmetic per array), the child references and the child count, and one wait for all of them.
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void load_node(const void *node, uint32_t onx, uint32_t ony, uint32_t onz, uint32_t ofx,
                                           uint32_t ofy, uint32_t ofz, u32x4 &NX, u32x4 &NY, u32x4 &NZ, u32x4 &FX,
                                           u32x4 &FY, u32x4 &FZ, u32x4 &refs, uint32_t &count) {
@@ -645,8 +646,21 @@ typedef const __attribute__((address_space(1))) uint32_t *global_u32;
 // deeper entries, or all of them without a shelf, live in private memory.
 constexpr int kLaneShelf = 32;
 struct LaneWalkAccel { const DstLeaf *leaves; const DstWideNode *wide; uint32_t n_leaves, root; };   // by value: registers
-__device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc, const RaySlab &slab, F3 o, F3 d,
-                                                    bool active, KBuf &buf_mem, uint32_t &cnt_mem, uint32_t *shelf) {
+static_assert(DST_GROUP <= 2, "the per-lane walk fetches a leaf group as at most two quad records");
+static_assert(sizeof(DstWideNode) == 128 && sizeof(DstLeaf) == 80, "the per-lane walk reads both as 16-byte words");
+// A value that is the same in every lane, moved to a scalar register (arguments of a real call arrive in vector ones).
+template <class T>
+__device__ __forceinline__ T *uniform_ptr(T *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<T *>(((uint64_t)hi << 32) | lo);
+}
+__device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc_in, const RaySlab &slab, F3 o, F3 d,
+                                                    bool active, KBuf &buf_mem, uint32_t &cnt_mem, uint32_t *shelf_in) {
+    const LaneWalkAccel acc = {uniform_ptr(acc_in.leaves), uniform_ptr(acc_in.wide),
+                               (uint32_t)__builtin_amdgcn_readfirstlane(acc_in.n_leaves),
+                               (uint32_t)__builtin_amdgcn_readfirstlane(acc_in.root)};
+    uint32_t *const shelf = uniform_ptr(shelf_in);
     // The caller's buffer is in memory (its address crosses the call): work on a register copy and store it once
     // at the end.  Left in memory, every leaf test re-read its 128 bytes per lane and every admission re-wrote them.
     KBuf buf = buf_mem;
@@ -655,49 +669,80 @@ __device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc, con
     fs.ix = slab.ix; fs.iy = slab.iy; fs.iz = slab.iz;
     fs.cnx = slab.nx - slab.wx; fs.cny = slab.ny - slab.wy; fs.cnz = slab.nz - slab.wz;
     fs.cfx = slab.nx + slab.wx; fs.cfy = slab.ny + slab.wy; fs.cfz = slab.nz + slab.wz;
-    // float index of this lane's near / far face arrays inside a wide node (lox 0, loy 4, loz 8, hix 12, hiy 16, hiz 20)
-    const uint32_t onx = slab.ix < 0.f ? 12u : 0u, ofx = 12u - onx;
-    const uint32_t ony = slab.iy < 0.f ? 16u : 4u, ofy = 20u - ony;
-    const uint32_t onz = slab.iz < 0.f ? 20u : 8u, ofz = 28u - onz;
+    const bool neg_x = slab.ix < 0.f, neg_y = slab.iy < 0.f, neg_z = slab.iz < 0.f;
     uint32_t stack[kLaneStack];
     int sp = 0;
     uint32_t ref = active ? acc.root : kWalkDone;
     uint32_t budget = 2u * acc.n_leaves + 8u;   // a well-formed hierarchy needs fewer steps; bounds the loop regardless
+    // A step of a lane is one dependent trip to memory: the lane's node (128 bytes) or its leaf group (two quad
+    // records of 80 bytes, consecutive) is requested whole - eight to ten 16-byte loads from one base address, whatever
+    // the lane is at - before anything is tested, so that lanes at nodes and lanes at leaf groups wait together,
+    // once.  (Left to the compiler, a quad came in three trips - corners A to C, then D and the normals behind the
+    // first edge test, then the surfel id behind the hit - and the lanes at leaf groups took theirs after the lanes
+    // at nodes had finished theirs.)
+    typedef const __attribute__((address_space(1))) v4f *global_v4f;
 #pragma unroll 1
     while (wave_ballot(ref != kWalkDone) != 0ull) {
         if (ref == kWalkDone) continue;
         uint32_t next = kWalkDone;
         bool have_next = false;
-        if (ref & DST_LEAF_BIT) {
-            const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
-#pragma unroll 1
-            for (uint32_t q = 0; q < count && first + q < acc.n_leaves; ++q) {
-                const global_f32 L = (global_f32)reinterpret_cast<const float *>(&acc.leaves[first + q]);
-                float t = 0.f;
-                uint32_t tri = 0u;
-                const bool hit = ray_quad(o, d, LD3(L, 0), LD3(L, 3), LD3(L, 6), LD3(L, 9), LD3(L, 12), LD3(L, 15), t, tri);
-                const uint64_t x = kb_pack(t, 2u * __float_as_uint(L[18]) + tri);
-                const bool adm = hit && (x < buf.e[kChunk - 1]);
-                if (adm) {
-                    cnt += 1u;
-                    kbuf_insert(buf, x, true);
+        const bool is_leaf = (ref & DST_LEAF_BIT) != 0u;
+        const uint32_t first = ref & DST_REF_FIRST_MASK, count = ((ref >> 28) & 7u) + 1u;
+        const bool good = is_leaf ? (first < acc.n_leaves) : (ref + 1u < acc.n_leaves);
+        if (good) {
+            const bool two = is_leaf && count > 1u && first + 1u < acc.n_leaves;
+            const global_v4f src = is_leaf ? (global_v4f)reinterpret_cast<const v4f *>(&acc.leaves[first])
+                                           : (global_v4f)reinterpret_cast<const v4f *>(&acc.wide[ref]);
+            // a node is 8 x 16 bytes; one quad is 5 (a leaf group of one quad asks for 8 as well: the array has spare
+            // records behind its last quad), two quads are 10
+            v4f r0 = src[0], r1 = src[1], r2 = src[2], r3 = src[3], r4 = src[4], r5 = src[5], r6 = src[6], r7 = src[7];
+            v4f r8 = {0.f, 0.f, 0.f, 0.f}, r9 = {0.f, 0.f, 0.f, 0.f};
+            if (two) {
+                r8 = src[8];
+                r9 = src[9];
+            }
+            // every value is in its registers here: nothing of the above may be requested later, behind a test
+            asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4));
+            asm volatile("" : "+v"(r5), "+v"(r6), "+v"(r7), "+v"(r8), "+v"(r9));
+            if (is_leaf) {
+                {
+                    float t = 0.f;
+                    uint32_t tri = 0u;
+                    const bool hit = ray_quad(o, d, f3(r0.x, r0.y, r0.z), f3(r0.w, r1.x, r1.y), f3(r1.z, r1.w, r2.x),
+                                              f3(r2.y, r2.z, r2.w), f3(r3.x, r3.y, r3.z), f3(r3.w, r4.x, r4.y), t, tri);
+                    const uint64_t x = kb_pack(t, 2u * __float_as_uint(r4.z) + tri);
+                    if (hit && (x < buf.e[kChunk - 1])) {
+                        cnt += 1u;
+                        kbuf_insert(buf, x, true);
+                    }
                 }
-            }
-        } else if (ref + 1u < acc.n_leaves) {
-            const global_f32 N = (global_f32)reinterpret_cast<const float *>(&acc.wide[ref]);
-            const global_u32 refs = (global_u32)reinterpret_cast<const uint32_t *>(&acc.wide[ref]) + 24;
-            const uint32_t n_child = refs[4];
-            const float tmax = kb_t(buf.e[kChunk - 1]);
-            uint32_t key[DST_WIDE], cref[DST_WIDE];
+                if (two) {
+                    float t = 0.f;
+                    uint32_t tri = 0u;
+                    const bool hit = ray_quad(o, d, f3(r5.x, r5.y, r5.z), f3(r5.w, r6.x, r6.y), f3(r6.z, r6.w, r7.x),
+                                              f3(r7.y, r7.z, r7.w), f3(r8.x, r8.y, r8.z), f3(r8.w, r9.x, r9.y), t, tri);
+                    const uint64_t x = kb_pack(t, 2u * __float_as_uint(r9.z) + tri);
+                    if (hit && (x < buf.e[kChunk - 1])) {
+                        cnt += 1u;
+                        kbuf_insert(buf, x, true);
+                    }
+                }
+                // (groups of more than two quads do not occur: DST_GROUP = 2; a longer one would lose its tail)
+            } else {
+                // lox r0, loy r1, loz r2, hix r3, hiy r4, hiz r5, child references r6, child count r7.x
+                const uint32_t n_child = __float_as_uint(r7.x);
+                const float tmax = kb_t(buf.e[kChunk - 1]);
+                uint32_t key[DST_WIDE], cref[DST_WIDE];
 #pragma unroll
-            for (int k = 0; k < DST_WIDE; ++k) {
-                float tn;
-                const uint64_t h = slab_hit_fast(fs, N[onx + k], N[ony + k], N[onz + k], N[ofx + k], N[ofy + k],
-                                                 N[ofz + k], tmax, tn);
-                const bool mine = ((h >> __lane_id()) & 1ull) != 0ull && (uint32_t)k < n_child;
-                key[k] = mine ? __float_as_uint(tn) : 0xFFFFFFFFu;   // entry distance (non-negative: bits order like the value)
-                cref[k] = refs[k];
-            }
+                for (int k = 0; k < DST_WIDE; ++k) {
+                    float tn;
+                    const uint64_t h = slab_hit_fast(fs, neg_x ? r3[k] : r0[k], neg_y ? r4[k] : r1[k], neg_z ? r5[k] : r2[k],
+                                                     neg_x ? r0[k] : r3[k], neg_y ? r1[k] : r4[k], neg_z ? r2[k] : r5[k],
+                                                     tmax, tn);
+                    const bool mine = ((h >> __lane_id()) & 1ull) != 0ull && (uint32_t)k < n_child;
+                    key[k] = mine ? __float_as_uint(tn) : 0xFFFFFFFFu;   // entry distance (non-negative: bits order like the value)
+                    cref[k] = __float_as_uint(r6[k]);
+                }
 #define CSWAP(a, b)                                                            \
     {                                                                          \
         const bool sw_ = key[b] < key[a];                                      \
@@ -705,20 +750,21 @@ __device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc, con
         const uint32_t ra_ = sw_ ? cref[b] : cref[a], rb_ = sw_ ? cref[a] : cref[b]; \
         key[a] = ka_; key[b] = kb_; cref[a] = ra_; cref[b] = rb_;              \
     }
-            CSWAP(0, 1) CSWAP(2, 3) CSWAP(0, 2) CSWAP(1, 3) CSWAP(1, 2)
+                CSWAP(0, 1) CSWAP(2, 3) CSWAP(0, 2) CSWAP(1, 3) CSWAP(1, 2)
 #undef CSWAP
-            // defer the farther children (farthest first), go on with the nearest
+                // defer the farther children (farthest first), go on with the nearest
 #pragma unroll
-            for (int k = DST_WIDE - 1; k >= 1; --k) {
-                if (key[k] != 0xFFFFFFFFu && sp < kLaneStack) {
-                    if (shelf != nullptr && sp < kLaneShelf) ((lds_u32)shelf)[sp * DST_WAVE + (int)__lane_id()] = cref[k];
-                    else stack[sp] = cref[k];
-                    ++sp;
+                for (int k = DST_WIDE - 1; k >= 1; --k) {
+                    if (key[k] != 0xFFFFFFFFu && sp < kLaneStack) {
+                        if (shelf != nullptr && sp < kLaneShelf) ((lds_u32)shelf)[sp * DST_WAVE + (int)__lane_id()] = cref[k];
+                        else stack[sp] = cref[k];
+                        ++sp;
+                    }
                 }
-            }
-            if (key[0] != 0xFFFFFFFFu) {
-                next = cref[0];
-                have_next = true;
+                if (key[0] != 0xFFFFFFFFu) {
+                    next = cref[0];
+                    have_next = true;
+                }
             }
         }
         if (!have_next && sp > 0) {
@@ -972,7 +1018,6 @@ __device__ __forceinline__ int table_slot(uint32_t *keys, uint32_t g) {
 constexpr int kStageCols = 16;                 // columns per tile
 constexpr int kStageStride = DST_WAVE + 1;     // floats per staged column: conflict-free writes and reads
 constexpr int kStageWords = kStageCols * kStageStride;
-typedef float v4f __attribute__((ext_vector_type(4)));
 template <int AUXM, bool DET>
 struct GradSink {
     const DstParams *p;
