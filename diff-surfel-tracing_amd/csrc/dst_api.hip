@@ -2,6 +2,7 @@
 // Replaces the pybind module and host launcher of the reference (ext.cpp, trace_surfels.cpp).
 #include "dst_internal.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -58,6 +59,7 @@ dst_ctx *dst_create(void) {
         delete ctx;
         return nullptr;
     }
+    if (const char *h = std::getenv("DST_HIERARCHY")) ctx->use_ploc = std::strcmp(h, "morton") != 0;
     if (dst_static_scratch_init(ctx) != DST_OK) {   // once per device, with that device current
         delete ctx;
         return nullptr;
@@ -71,6 +73,7 @@ void dst_destroy(dst_ctx *ctx) {
     if (ctx->bounds) (void)hipFree(ctx->bounds);
     if (ctx->core_box) (void)hipFree(ctx->core_box);
     if (ctx->bounds_host) (void)hipHostFree(ctx->bounds_host);
+    if (ctx->ploc_host) (void)hipHostFree(ctx->ploc_host);
     delete ctx;
 }
 
@@ -171,6 +174,8 @@ int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info) {
     info->builds = ctx->builds;
     info->refits = ctx->refits;
     info->key_levels = ctx->fine_keys ? 2u : 1u;
+    info->agglomerated = ctx->agglomerated ? 1u : 0u;
+    info->depth = ctx->hierarchy_depth;
     return DST_OK;
 }
 

@@ -95,6 +95,12 @@ struct dst_ctx {
     uint32_t built_vertices = 0;   // rows of the vertex buffer the stored quad ids were validated against
     bool canonical = false;        // the build's quads were rows 4g..4g+3 of the vertex buffer, in that order
     uint32_t builds = 0, refits = 0;
+    bool use_ploc = true;          // builds make the hierarchy by agglomeration (DST_HIERARCHY=morton in the environment: Karras)
+    bool ploc_refused = false;     // an agglomerated hierarchy came out too deep: Morton hierarchy for good
+    bool agglomerated = false;     // how the current structure's hierarchy was made
+    uint32_t hierarchy_depth = 0;  // nodes above its deepest leaf (agglomerated hierarchies; 0: not measured)
+    uint32_t *ploc_state = nullptr, *ploc_host = nullptr;   // device / pinned host: counters of the agglomeration
+    uint32_t ploc_blocks = 0;
     DstNode *nodes = nullptr;
     DstWideNode *wide = nullptr;
     DstLeaf *leaves = nullptr;

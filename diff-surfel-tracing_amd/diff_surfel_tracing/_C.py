@@ -44,7 +44,7 @@ class DstAccelInfo(C.Structure):
     _fields_ = [("n_surfels", C.c_uint32), ("n_internal", C.c_uint32), ("root", C.c_uint32),
                 ("node_bytes", C.c_uint32), ("leaf_bytes", C.c_uint32), ("scene_lo", C.c_float * 3),
                 ("scene_hi", C.c_float * 3), ("max_abs", C.c_float), ("builds", C.c_uint32), ("refits", C.c_uint32),
-                ("key_levels", C.c_uint32)]
+                ("key_levels", C.c_uint32), ("agglomerated", C.c_uint32), ("depth", C.c_uint32)]
 
 
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",

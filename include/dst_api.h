@@ -136,6 +136,12 @@ typedef struct DstAccelInfo {
     uint32_t key_levels;   /* 1: the builds sort 30-bit Morton keys; 2: 60-bit keys in two levels, which a context goes
                               over to, for good, when a build finds more than three quarters of the surfels sharing
                               their cell of the 1024^3 grid with a neighbour (surfels far outside a compact scene) */
+    uint32_t agglomerated; /* 1: the hierarchy was made by merging neighbouring clusters of quads by the surface of their
+                              union, starting from the Morton order (what builds do by default); 0: read off the Morton
+                              codes alone (scenes of fewer than 64 surfels, DST_HIERARCHY=morton in the environment when
+                              the context was created, or a context whose agglomerated hierarchy came out deeper than
+                              the walks' stacks allow) */
+    uint32_t depth;        /* nodes above the deepest leaf of an agglomerated hierarchy (0: not measured) */
 } DstAccelInfo;
 
 /* Create / destroy the tracer state on the current HIP device.
@@ -149,7 +155,8 @@ void dst_destroy(dst_ctx *ctx);
  * int32 with rows 2g and 2g+1 forming surfel g's quad and sharing an edge
  * (rows [a,b,c] and [b,c,d]).  A refit reuses the topology of the last build:
  * n_triangles must be unchanged and `triangles` is not read.  A build waits
- * for the stream once (it reads back a validity flag); a refit does not.
+ * for the stream a few times (it reads back a validity flag and, while it merges
+ * clusters into the hierarchy, how many are left); a refit does not.
  * Replaces BuildAccelerationStructure (trace_surfels.cpp:36-159). */
 int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, const int32_t *triangles,
                     uint32_t n_triangles, int rebuild, void *stream);
@@ -192,7 +199,8 @@ const char *dst_last_error(dst_ctx *ctx);
 /* Introspection for tests: shape of the BVH, and copies of its arrays to HOST
  * buffers (each may be NULL to skip).  nodes: n_internal*node_bytes, leaves:
  * n_surfels*leaf_bytes, node_parent: n_internal uint32, leaf_parent: n_surfels
- * uint32, sorted_keys: n_surfels uint32 Morton codes in leaf order.  Waits for the stream. */
+ * uint32, sorted_keys: the n_surfels uint32 Morton codes in ascending order (the leaf order of a hierarchy read off
+ * the codes; the order an agglomeration starts from).  Waits for the stream. */
 int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info);
 int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_parent, uint32_t *leaf_parent,
                        uint32_t *sorted_keys, void *stream);

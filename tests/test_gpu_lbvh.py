@@ -33,9 +33,34 @@ def download(tracer):
     return info, nodes[: n - 1], leaves, npar[: n - 1], lpar, keys
 
 
+def own_tracer(hierarchy):
+    """A tracer of its own whose builds make the hierarchy by agglomeration (the default) or read it off the Morton
+    codes (`DST_HIERARCHY=morton` in the environment when the context is created)."""
+    import os
+
+    import diff_surfel_tracing as dst
+    saved = os.environ.get("DST_HIERARCHY")
+    try:
+        if hierarchy == "morton":
+            os.environ["DST_HIERARCHY"] = "morton"
+        else:
+            os.environ.pop("DST_HIERARCHY", None)
+        return dst.SurfelTracer()
+    finally:
+        if saved is None:
+            os.environ.pop("DST_HIERARCHY", None)
+        else:
+            os.environ["DST_HIERARCHY"] = saved
+
+
 def check_tree(info, nodes, leaves, npar, lpar, keys, vertices):
     n = info.n_surfels
-    assert (np.diff(keys.astype(np.int64)) >= 0).all()                 # Morton order
+    assert (np.diff(keys.astype(np.int64)) >= 0).all()                 # the sort's result: Morton codes ascending
+    for i in range(n - 1):                                             # a node's leaves are consecutive; the numbering
+        f, l, c0, c1 = (int(nodes[k][i]) for k in ("first", "last", "c0", "c1"))   # of its children follows from them
+        split = c0 & ~LEAF
+        assert f <= split < l and (c1 & ~LEAF) == split + 1
+        assert bool(c0 & LEAF) == (split == f) and bool(c1 & LEAF) == (split + 1 == l)
     assert sorted(leaves["g"].tolist()) == list(range(n))              # every surfel exactly once
     V = vertices.reshape(n, 4, 3)
     for name, k in (("A", 0), ("B", 1), ("C", 2), ("D", 3)):
@@ -87,8 +112,11 @@ def check_tree(info, nodes, leaves, npar, lpar, keys, vertices):
     return maxdepth
 
 
-@pytest.mark.parametrize("maker,P", [(S.scene_cube, 5000), (S.scene_room, 20000), (S.scene_cube, 2), (S.scene_cube, 1025)])
-def test_tree_invariants_after_build_and_refit(tracer, maker, P):
+@pytest.mark.parametrize("hierarchy", ["agglomerated", "morton"])
+@pytest.mark.parametrize("maker,P", [(S.scene_cube, 5000), (S.scene_room, 20000), (S.scene_cube, 2), (S.scene_cube, 1025),
+                                     (S.scene_cube, 64), (S.scene_room, 3333)])
+def test_tree_invariants_after_build_and_refit(maker, P, hierarchy):
+    tracer = own_tracer(hierarchy)
     sc = maker(P=P, seed=1)
     v, f = sc["vertices"].cuda(), sc["faces"].cuda()
     tracer.build_acceleration_structure(v, f, True)
@@ -98,7 +126,9 @@ def test_tree_invariants_after_build_and_refit(tracer, maker, P):
     np.testing.assert_allclose(list(info.scene_lo), cen.min(0), rtol=0, atol=0)
     np.testing.assert_allclose(list(info.scene_hi), cen.max(0), rtol=0, atol=0)
     assert info.max_abs == float(sc["vertices"].abs().max())
-    check_tree(info, *arrs, sc["vertices"].numpy())
+    assert info.agglomerated == int(hierarchy == "agglomerated" and P >= 64)
+    depth = check_tree(info, *arrs, sc["vertices"].numpy())
+    assert info.depth == (depth + 1 if info.agglomerated else 0)       # nodes above the deepest leaf
     moved = S.perturb_means(sc, 1, frac=0.5, sigma=0.2)
     tracer.build_acceleration_structure(moved["vertices"].cuda(), f, False)
     info2, *arrs2 = download(tracer)
@@ -108,8 +138,11 @@ def test_tree_invariants_after_build_and_refit(tracer, maker, P):
     assert info2.refits >= 1
 
 
-def test_duplicate_positions_give_a_bounded_tree(tracer):
-    """All centroids in one Morton cell: the hierarchy falls back to index bits and stays balanced."""
+@pytest.mark.parametrize("hierarchy", ["agglomerated", "morton"])
+def test_duplicate_positions_give_a_bounded_tree(hierarchy):
+    """All centroids in one Morton cell: the Morton hierarchy falls back to index bits and stays balanced; the
+    agglomeration pairs the quads by their boxes whatever their order."""
+    tracer = own_tracer(hierarchy)
     P = 4096
     sc = S.scene_cube(P=P, seed=2)
     sc["means3D"] = torch.zeros(P, 3)
@@ -118,6 +151,21 @@ def test_duplicate_positions_give_a_bounded_tree(tracer):
     info, *arrs = download(tracer)
     depth = check_tree(info, *arrs, sc["vertices"].numpy())
     assert depth <= 44   # 30 key bits + 12 index bits
+
+
+def test_identical_quads_pair_up(tracer):
+    """20000 copies of one surfel (and a few others): every union has the same surface, and the agglomeration's order
+    on equal pairs must still merge half of them per round and end in a hierarchy a dozen or so levels deep."""
+    P = 20000
+    sc = S.scene_cube(P=P, seed=3)
+    for k in ("means3D", "scales", "rotations"):
+        sc[k][:P - 50] = sc[k][0]
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    own = own_tracer("agglomerated")
+    own.build_acceleration_structure(sc["vertices"].cuda(), sc["faces"].cuda(), True)
+    info, *arrs = download(own)
+    assert info.agglomerated == 1
+    assert check_tree(info, *arrs, sc["vertices"].numpy()) <= 24
 
 
 def _with_far_surfels(sc, factor, k=5, seed=4):
@@ -131,12 +179,12 @@ def _with_far_surfels(sc, factor, k=5, seed=4):
     return out
 
 
-def test_surfels_far_outside_a_compact_scene_switch_the_builds_to_two_level_keys():
+@pytest.mark.parametrize("hierarchy", ["agglomerated", "morton"])
+def test_surfels_far_outside_a_compact_scene_switch_the_builds_to_two_level_keys(hierarchy):
     """A few surfels 2000 scene radii away stretch the 1024^3 Morton grid until the scene itself fills one cell: the
     build notices (nearly all neighbours in Morton order share their cell), builds again with 60-bit keys in two
     levels and keeps them for the context's later builds.  The structure obeys the same invariants either way."""
-    import diff_surfel_tracing as dst
-    own = dst.SurfelTracer()
+    own = own_tracer(hierarchy)
     sc = S.scene_cube(P=20000, seed=8)
     own.build_acceleration_structure(sc["vertices"].cuda(), sc["faces"].cuda(), True)
     info, *arrs = download(own)
@@ -163,9 +211,9 @@ def test_two_level_keys_are_given_up_when_the_hierarchy_gets_too_deep():
     """Sixty surfels that each peel one bit off the 60-bit key (one per axis and scale, down to a millionth of the
     extent) in front of 16384 surfels at one point, and a uniform cloud that keeps the box of the keys at full
     size: with two-level keys the deepest leaf lies 74 nodes down, more than the walks' stacks are sized for.  The
-    build measures that and returns to one-level keys for good."""
-    import diff_surfel_tracing as dst
-    own = dst.SurfelTracer()
+    build measures that and returns to one-level keys for good.  (Hierarchies read off the Morton codes: an agglomerated
+    one does not follow the key bits down.)"""
+    own = own_tracer("morton")
     pts = [[0.0, 0.0, 0.0]] * 16384
     pts += (torch.rand(4096, 3, generator=torch.Generator().manual_seed(3)) * 1.2).tolist()
     for k in range(20):
