@@ -261,6 +261,23 @@ def run_workload(key, steps, warmup, main, args):
     torch.cuda.synchronize()
     bwd_retrace_ms = sum(a.elapsed_time(b) for a, b in alt) / n_alt
 
+    # --- the same step with the SH coefficients read from their binary16 copy (DST_FLAG_SH_HALF; the copy is made by
+    # a packing kernel in front of every trace, timed on its own)
+    sh_half = None
+    if main:
+        pack_ms = median(lambda: _C.pack_sh_half(g["shs"]))
+        ctx.sh_half = True
+        alt_f = [(ev(), ev()) for _ in range(n_alt)]
+        alt_b = [(ev(), ev()) for _ in range(n_alt)]
+        step()
+        for k in range(n_alt):
+            step(alt_f[k], alt_b[k])
+        torch.cuda.synchronize()
+        ctx.sh_half = False
+        sh_half = {"fwd_kernel_ms": round(sum(a.elapsed_time(b) for a, b in alt_f) / n_alt, 4),
+                   "bwd_kernel_ms": round(sum(a.elapsed_time(b) for a, b in alt_b) / n_alt, 4),
+                   "pack_ms": round(pack_ms, 4)}
+
     A_fwd = R * FWD_RAY + n_proc * FWD_PROC + n_con * FWD_CON
     A_bwd = R * BWD_RAY + n_proc * BWD_PROC + n_con * BWD_CON
     A_total = A_fwd + A_bwd + PER_SURFEL_INIT * P
@@ -298,6 +315,8 @@ def run_workload(key, steps, warmup, main, args):
         "reference_equivalent_hbm_frac": round(A_total / (ms_per_step * 1e-3) / (HBM_PEAK_GBS * 1e9), 5),
         "roofline_kernels": per_kernel,
     }
+    if sh_half is not None:
+        result["sh_half"] = sh_half
     if geo_ms:
         result["geometry_update_ms_per_frame"] = round(sum(geo_ms) / len(geo_ms), 4)
         result["frame_loop"] = ("%d views, structure built once and refitted before each" % len(frames) if wl.get("views")

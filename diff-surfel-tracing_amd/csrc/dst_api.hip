@@ -35,8 +35,9 @@ int check_common(dst_ctx *ctx, const DstParams *p) {
                         "vertices, background, means3D, opacities, scales and rotations are required");
     if ((p->flags & DST_FLAG_DETERMINISTIC) && !p->det_workspace)
         return dst_fail(ctx, DST_E_INVALID, "the deterministic mode needs det_workspace");
-    if (p->flags & ~(DST_FLAG_DETERMINISTIC | DST_FLAG_DISTORTION))
+    if (p->flags & ~(DST_FLAG_DETERMINISTIC | DST_FLAG_DISTORTION | DST_FLAG_SH_HALF))
         return dst_fail(ctx, DST_E_INVALID, "unknown bits in flags");
+
     if (p->hit_record && (reinterpret_cast<uintptr_t>(p->hit_record) & 7u))
         return dst_fail(ctx, DST_E_INVALID, "hit_record must be 8-byte aligned");
     if (p->H > 0 && p->W > 0 &&
@@ -140,6 +141,8 @@ int dst_trace_forward(dst_ctx *ctx, const DstParams *p, void *stream) {
     int rc = check_common(ctx, p);
     if (rc) return rc;
     if (p->training && !p->a_weights) return dst_fail(ctx, DST_E_INVALID, "training needs a_weights");
+    if ((p->flags & DST_FLAG_SH_HALF) && (!p->shs || !p->shs_half))
+        return dst_fail(ctx, DST_E_INVALID, "DST_FLAG_SH_HALF needs shs and its binary16 copy shs_half");
     return dst_launch_trace(ctx, *p, false, (hipStream_t)stream);
 }
 
@@ -156,6 +159,12 @@ int dst_trace_backward(dst_ctx *ctx, const DstParams *p, void *stream) {
     if (p->shs && !p->dL_dshs) return dst_fail(ctx, DST_E_INVALID, "dL_dshs missing");
     if (p->others_precomp && !p->dL_dothers) return dst_fail(ctx, DST_E_INVALID, "dL_dothers missing");
     return dst_launch_trace(ctx, *p, true, (hipStream_t)stream);
+}
+
+int dst_pack_sh_half(const float *shs, uint16_t *out, uint64_t n_values, void *stream) {
+    if (n_values == 0) return DST_OK;
+    if (!shs || !out) return DST_E_INVALID;
+    return dst_launch_pack_half(shs, out, n_values, (hipStream_t)stream);
 }
 
 int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info) {

@@ -150,6 +150,7 @@ void dst_sort_pairs(uint32_t *keys[2], uint32_t *vals[2], uint32_t *tile_hist, u
 size_t dst_sort_hist_elems(uint32_t n);
 // trace.hip
 int dst_launch_trace(dst_ctx *ctx, const DstParams &p, bool backward, hipStream_t stream);
+int dst_launch_pack_half(const float *src, uint16_t *dst, uint64_t n, hipStream_t stream);
 
 static inline int dst_fail(dst_ctx *ctx, int code, const std::string &msg) {
     if (ctx) ctx->err = msg;

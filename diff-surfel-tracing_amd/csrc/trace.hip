@@ -12,6 +12,8 @@
 // gradient algebra, which feeds no decision, allows fused multiply-adds.
 #include "dst_internal.h"
 
+#include <algorithm>
+
 namespace {
 
 constexpr int kChunk = 16;
@@ -89,11 +91,42 @@ __device__ __forceinline__ void quat_rows(const float q0, const float q1, const 
     R[2] = f3(2.f * (x * z + w * y), 2.f * (y * z - w * x), 1.f - 2.f * (x * x + y * y));
 }
 
+// Where a surfel's SH coefficients come from: the caller's fp32 tensor, or (DST_FLAG_SH_HALF) its binary16 copy,
+// widened to fp32 as it is read - the arithmetic after that is the same fp32 sequence either way.
+struct ShF32 {
+    const float *p;
+    __device__ __forceinline__ float operator()(int k) const { return p[k]; }
+};
+struct ShF16 {
+    const uint16_t *p;
+    __device__ __forceinline__ float operator()(int k) const { return (float)__builtin_bit_cast(_Float16, p[k]); }
+};
+// The first `n_halves` binary16 coefficients of a surfel as 16-byte loads (rows of 16 coefficients x 3 channels are 96
+// bytes, so every row starts on a 16-byte boundary when the tensor does), kept in registers.
+struct ShF16Row {
+    uint32_t w[24];
+    __device__ __forceinline__ void load(const uint16_t *row, int n_halves) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(row);
+#pragma unroll
+        for (int k = 0; k < 6; ++k) {
+            if (8 * k < n_halves) {
+                const uint4 v = src[k];
+                w[4 * k] = v.x; w[4 * k + 1] = v.y; w[4 * k + 2] = v.z; w[4 * k + 3] = v.w;
+            } else {
+                w[4 * k] = w[4 * k + 1] = w[4 * k + 2] = w[4 * k + 3] = 0u;
+            }
+        }
+    }
+    __device__ __forceinline__ float operator()(int k) const {
+        const uint32_t word = w[k >> 1];
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)((k & 1) ? (word >> 16) : (word & 0xFFFFu)));
+    }
+};
+
 // SH colour of one surfel in direction d (reference forward.cu:18-58); clamp flags for backward.
-__device__ __forceinline__ F3 sh_color(int deg, const float *__restrict__ sh, F3 d, bool (&neg)[3]) {
-#define SHC(j) f3(sh[3 * (j)], sh[3 * (j) + 1], sh[3 * (j) + 2])
-
-
+template <class SH>
+__device__ __forceinline__ F3 sh_color(int deg, const SH &sh, F3 d, bool (&neg)[3]) {
+#define SHC(j) f3(sh(3 * (j)), sh(3 * (j) + 1), sh(3 * (j) + 2))
     F3 r = SH0 * SHC(0);
     if (deg > 0) {
         float x = d.x, y = d.y, z = d.z;
@@ -111,11 +144,22 @@ __device__ __forceinline__ F3 sh_color(int deg, const float *__restrict__ sh, F3
             }
         }
     }
+#undef SHC
     r = f3(r.x + 0.5f, r.y + 0.5f, r.z + 0.5f);
     neg[0] = r.x < 0.f;
     neg[1] = r.y < 0.f;
     neg[2] = r.z < 0.f;
     return f3(r.x > 0.f ? r.x : 0.f, r.y > 0.f ? r.y : 0.f, r.z > 0.f ? r.z : 0.f);
+}
+// The colour from the binary16 copy of the coefficients (DST_FLAG_SH_HALF).
+__device__ __forceinline__ F3 sh_color_half(const DstParams &p, int g, F3 d, bool (&neg)[3]) {
+    const uint16_t *row = p.shs_half + (size_t)g * p.M * 3;
+    if ((p.M & 7) == 0 && p.M <= 16 && (reinterpret_cast<uintptr_t>(p.shs_half) & 15u) == 0u) {
+        ShF16Row r;
+        r.load(row, 3 * (p.D + 1) * (p.D + 1));
+        return sh_color(p.D, r, d, neg);
+    }
+    return sh_color(p.D, ShF16{row}, d, neg);
 }
 
 // ---- ray / quad -----------------------------------------------------------------------------------------
@@ -1174,9 +1218,10 @@ struct LastShHit {
     unsigned long long t0, t_alg, t_sh;
 #endif
 };
-__device__ __forceinline__ F3 sh_direction_gradient(int deg, const float *__restrict__ sh, F3 rd, F3 gc) {
+template <class SH>
+__device__ __forceinline__ F3 sh_direction_gradient(int deg, const SH &sh, F3 rd, F3 gc) {
 #pragma clang fp contract(fast)
-    auto S = [&](int j) { return f3(sh[3 * j], sh[3 * j + 1], sh[3 * j + 2]); };
+    auto S = [&](int j) { return f3(sh(3 * j), sh(3 * j + 1), sh(3 * j + 2)); };
     F3 ddx = f3(0, 0, 0), ddy = f3(0, 0, 0), ddz = f3(0, 0, 0);
     const float x = rd.x, y = rd.y, z = rd.z;
     if (deg > 0) {
@@ -1642,7 +1687,10 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
                     }
                 } else if (p.colors_precomp == nullptr) {
                     sh = p.shs + (size_t)g * p.M * 3;
-                    F3 c = sh_color(p.D, sh, rd, neg);
+                    // (the binary16 source lives in the forward kernels that carry the rarely used options; a backward
+                    // trace is given the widened values as shs)
+                    const F3 c = (!BWD && DET && (p.flags & DST_FLAG_SH_HALF)) ? sh_color_half(p, g, rd, neg)
+                                                                              : sh_color(p.D, ShF32{sh}, rd, neg);
                     col[0] = c.x; col[1] = c.y; col[2] = c.z;
                 } else {
                     col[0] = p.colors_precomp[3 * (size_t)g];
@@ -1733,7 +1781,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
         rv.dir[bounce] = (rv.dir[bounce] & kRecDirBlockMask) | (min(rec_chunks, 63u) << kRecDirBlockBits);
     STAT(if (BWD) { ws.nodes += last_sh.t_alg; ws.leaves += last_sh.t_sh; })
     if (BWD && p.colors_precomp == nullptr && last_sh.any)
-        g_rd = sh_direction_gradient(p.D, p.shs + (size_t)last_sh.g * p.M * 3, rd, last_sh.gc);
+        g_rd = sh_direction_gradient(p.D, ShF32{p.shs + (size_t)last_sh.g * p.M * 3}, rd, last_sh.gc);
     run.T = Tp;
 }
 
@@ -2202,6 +2250,11 @@ __global__ void k_ray_keys(const float *__restrict__ ray_o, const float *__restr
     vals[r] = r;
 }
 
+__global__ void k_pack_half(const float *__restrict__ src, uint16_t *__restrict__ dst, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x)
+        dst[i] = __builtin_bit_cast(uint16_t, (_Float16)src[i]);   // round to nearest even
+}
+
 struct TileGrid {
     int tw_log2, th_log2;
     uint32_t tiles_x, tiles_y, btiles_x, btiles_y;
@@ -2280,6 +2333,12 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
 }
 
 }  // namespace
+
+int dst_launch_pack_half(const float *src, uint16_t *dst, uint64_t n, hipStream_t stream) {
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + 255u) / 256u, 4096u);
+    hipLaunchKernelGGL(k_pack_half, dim3(blocks), dim3(256), 0, stream, src, dst, n);
+    return hipGetLastError() == hipSuccess ? DST_OK : DST_E_DEVICE;
+}
 
 uint64_t dst_det_workspace_words(int32_t P, int32_t aux, int backward) {
     if (P <= 0 || aux < 1 || aux > DST_MAX_AUX) return 0;

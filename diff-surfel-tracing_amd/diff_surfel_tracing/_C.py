@@ -19,6 +19,7 @@ MAX_AUX_CHANNELS = 8
 MAX_TRACE_DEPTH = 3
 FLAG_DETERMINISTIC = 1
 FLAG_DISTORTION = 2
+FLAG_SH_HALF = 4
 
 _FP = C.c_void_p
 
@@ -37,6 +38,7 @@ class DstParams(C.Structure):
         + [(n, _FP) for n in ("dL_drgb", "dL_ddpt", "dL_dacc", "dL_ddist", "dL_dnorm", "dL_daux")]
         + [(n, _FP) for n in ("dL_dray_o", "dL_dray_d", "dL_dmeans3D", "dL_dgrads3D", "dL_dshs", "dL_dcolors",
                               "dL_dothers", "dL_dopacities", "dL_dscales", "dL_drotations")]
+        + [("shs_half", _FP)]
     )
 
 
@@ -50,7 +52,7 @@ class DstAccelInfo(C.Structure):
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
            "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params",
            "dst_hit_record_layout", "dst_refit_accel_static", "dst_refit_from_surfels",
-           "dst_det_workspace_words")
+           "dst_det_workspace_words", "dst_pack_sh_half")
 
 _lib = None
 
@@ -80,6 +82,7 @@ def load_library():
     L.dst_accel_download.argtypes = [C.c_void_p] * 7
     L.dst_det_workspace_words.restype = C.c_uint64
     L.dst_det_workspace_words.argtypes = [C.c_int32, C.c_int32, C.c_int]
+    L.dst_pack_sh_half.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
     L.dst_version.restype = C.c_char_p
     L.dst_sizeof_params.restype = C.c_size_t
     L.dst_hit_record_layout.restype = C.c_uint64
@@ -204,6 +207,7 @@ class OptiXStateWrapper:
         self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
         self.gradient_rows = True           # backward sums per-surfel gradients in one row per surfel first (faster)
         self.distortion = False             # True: the dist output carries the 2DGS depth distortion (else zeros)
+        self.sh_half = False                # True: the traces read the SH coefficients from a binary16 copy
         self._record_pool = []              # free storages (int64 tensors)
         self._record_events = {}            # id(storage) -> event recorded when the storage came back
         self._record_fixed = False          # True: only caller-provided storage is used, nothing is allocated
@@ -339,6 +343,24 @@ def refit_from_surfels(ctx, means3D, scales, rotations, vertices_out=None):
     return vertices_out
 
 
+def pack_sh_half(shs):
+    """binary16 copy of an fp32 CUDA tensor of SH coefficients (dst_pack_sh_half: round to nearest even)."""
+    shs = _cuda_f32(shs, "shs")
+    out = torch.empty(shs.shape, dtype=torch.float16, device=shs.device)
+    rc = load_library().dst_pack_sh_half(shs.data_ptr(), out.data_ptr(), shs.numel(), _stream())
+    if rc != 0:
+        raise RuntimeError("dst_pack_sh_half failed (status %d)" % rc)
+    return out
+
+
+def _use_sh_half(ctx, p, keep):
+    """With `ctx.sh_half` set and SH coefficients given: pack them and point the launch parameters at the copy."""
+    if getattr(ctx, "sh_half", False) and keep["shs"].numel() != 0:
+        keep["shs_half"] = pack_sh_half(keep["shs"])
+        p.shs_half = keep["shs_half"].data_ptr()
+        p.flags |= FLAG_SH_HALF
+
+
 def _common_params(ray_o, ray_d, vertices, background, means3D, shs, degree, colors_precomp, others_precomp,
                    opacities, scales, scale_modifier, rotations, max_trace_depth, specular_threshold,
                    start_from_first):
@@ -405,6 +427,7 @@ def trace_surfels(ctx, training, start_from_first, ray_o, ray_d, vertices, backg
         p.flags, p.det_workspace = FLAG_DETERMINISTIC, det_ws.data_ptr()
     if getattr(ctx, "distortion", False):
         p.flags |= FLAG_DISTORTION
+    _use_sh_half(ctx, p, keep)
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_forward(ctx.handle, C.byref(p), _stream()))
@@ -471,6 +494,10 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
         # the per-surfel gradients are summed in rows of one buffer first (a surfel's columns side by side)
         det_ws = torch.zeros(load_library().dst_det_workspace_words(P, p.aux, 1), dtype=torch.float32, device=dev)
         p.grad_rows = det_ws.data_ptr()
+    if getattr(ctx, "sh_half", False) and keep["shs"].numel() != 0:
+        # the backward trace reads fp32 coefficients: the values the forward trace used
+        keep["shs"] = pack_sh_half(keep["shs"]).float()
+        p.shs = keep["shs"].data_ptr()
     if events is not None:
         events[0].record()
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))

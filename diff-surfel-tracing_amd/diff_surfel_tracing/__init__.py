@@ -160,6 +160,18 @@ class SurfelTracer(nn.Module):
     def distortion(self, value: bool) -> None:
         self.optix_context.distortion = bool(value)
 
+    @property
+    def sh_half(self) -> bool:
+        """Extension (not in the reference): when set, every trace packs the SH coefficients to binary16 (round to
+        nearest even) and the kernels read that copy, widening to fp32 as they go - half the bytes of the largest
+        per-hit gather.  Results are exactly those of `shs.half().float()`; the gradient of `shs` is that of the fp32
+        coefficients (the rounding is not differentiated)."""
+        return self.optix_context.sh_half
+
+    @sh_half.setter
+    def sh_half(self, value: bool) -> None:
+        self.optix_context.sh_half = bool(value)
+
     def build_acceleration_structure(self, vertices: torch.Tensor, triangles: torch.Tensor, rebuild: bool = 1):
         """Build (`rebuild` true) or refit in place the BVH over the surfel quads `vertices` (4P,3), `triangles` (2P,3)."""
         return _C.build_acceleration_structure(self.optix_context, vertices, triangles, rebuild)

@@ -41,6 +41,13 @@ enum {
                                    * without the flag.  No gradient flows from it (the reference's backward never reads
                                    * dL_ddist either). */
 
+#define DST_FLAG_SH_HALF 4u       /* forward: the trace reads the SH coefficients from DstParams.shs_half, a binary16 copy
+                                   * of shs (made with dst_pack_sh_half), and widens them to fp32 as they are read: half
+                                   * the bytes of the largest per-hit gather; results are those of fp32 coefficients that
+                                   * hold the rounded values, bit for bit.  A backward trace ignores the flag and reads
+                                   * shs: give it the values the forward trace used (the binary16 values, widened); its
+                                   * dL_dshs is then the gradient with respect to those.  No counterpart in the reference. */
+
 #define DST_MAX_AUX 8        /* auxiliary channels per surfel (reference AUX_CHANNELS = 2) */
 #define DST_MAX_TRACE_DEPTH 3 /* bounces after the primary ray (reference MAX_TRACE_DEPTH = 1) */
 #define DST_STATIC_REFIT_MAX_SURFELS (1u << 21) /* largest structure dst_refit_accel_static serves */
@@ -122,6 +129,9 @@ typedef struct DstParams {
     float *dL_dopacities;         /* (P,1) */
     float *dL_dscales;            /* (P,2) */
     float *dL_drotations;         /* (P,4) */
+    /* forward, DST_FLAG_SH_HALF: binary16 copy of shs, same shape (P,M,3); NULL otherwise (last in the block: the
+     * kernels fetch their arguments in groups, and a field in the middle would move the others) */
+    const uint16_t *shs_half;
 } DstParams;
 
 /* Shape of the current acceleration structure, for tests and tools. */
@@ -214,6 +224,11 @@ uint64_t dst_hit_record_layout(int32_t H, int32_t W, int32_t mtd_alloc, uint32_t
 /* Words (8 bytes each) of DstParams.det_workspace for a forward (backward = 0: one per surfel) or a backward
  * call (one per surfel and gradient column: 16 + aux table columns + 48 SH columns). */
 uint64_t dst_det_workspace_words(int32_t P, int32_t aux, int backward);
+
+/* fp32 -> binary16 (round to nearest even, overflow to infinity) of `n_values` SH coefficients: out[i] = half(shs[i]).
+ * Device pointers; stream-ordered, no wait.  Makes DstParams.shs_half for DST_FLAG_SH_HALF.  No counterpart in the
+ * reference, whose SH coefficients are fp32 (optix_tracer/forward.cu:265-268). */
+int dst_pack_sh_half(const float *shs, uint16_t *out, uint64_t n_values, void *stream);
 
 /* Library version string, and sizeof(DstParams) as compiled (lets a foreign-language binding
  * verify its own struct layout before the first launch). */
