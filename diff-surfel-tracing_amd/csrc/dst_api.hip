@@ -99,6 +99,12 @@ int dst_build_accel(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, co
         if (n_vertices < ctx->built_vertices)
             return dst_fail(ctx, DST_E_TOPOLOGY, "refit (rebuild=False) with fewer vertices than the build indexed");
     }
+    if (rebuild && (ctx->fine_keys_refused || ctx->ploc_refused) && ++ctx->refused_builds >= 16u) {
+        // a refusal (two-level keys or an agglomerated hierarchy came out too deep for one scene) is not for ever:
+        // every sixteenth build tries again
+        ctx->fine_keys_refused = ctx->ploc_refused = false;
+        ctx->refused_builds = 0u;
+    }
     return dst_lbvh_build(ctx, vertices, n_vertices, triangles, P, rebuild != 0, (hipStream_t)stream);
 }
 
@@ -180,6 +186,11 @@ int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info) {
         info->scene_hi[a] = ctx->scene_hi[a];
     }
     info->max_abs = ctx->max_abs;
+    if (ctx->bounds != nullptr && ctx->bounds_host != nullptr) {
+        // what refits and traces have left on the device since the build (waits for the device)
+        DST_HIP(ctx, hipMemcpy(ctx->bounds_host, ctx->bounds, sizeof(DstBounds), hipMemcpyDeviceToHost));
+        std::memcpy(&info->max_abs, &ctx->bounds_host->max_abs, 4);
+    }
     info->builds = ctx->builds;
     info->refits = ctx->refits;
     info->key_levels = ctx->fine_keys ? 2u : 1u;

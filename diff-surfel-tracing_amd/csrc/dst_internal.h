@@ -91,6 +91,7 @@ struct dst_ctx {
     uint32_t capacity = 0;      // surfels the buffers can hold
     bool fine_keys = false;     // builds sort two-level Morton keys (set when a build finds the one-level grid too coarse)
     bool fine_keys_refused = false;   // a build with two-level keys came out too deep for the walks' stacks
+    uint32_t refused_builds = 0;      // builds since a refusal (the sixteenth tries again)
     bool built = false;
     uint32_t built_vertices = 0;   // rows of the vertex buffer the stored quad ids were validated against
     bool canonical = false;        // the build's quads were rows 4g..4g+3 of the vertex buffer, in that order

@@ -506,8 +506,11 @@ struct WalkList {
 
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
 // to its origin, 0 < t < 1e16) and the number of admissions.  Wave-uniform control flow: nodes and quads
-// are fetched once per wave, the stack is two VGPRs addressed by lane (128 entries: the binary hierarchy
-// is at most 62 levels deep, a 4-wide step goes down two of them and defers at most three children: 96).
+// are fetched once per wave, the stack is two VGPRs addressed by lane.  128 entries are enough by construction:
+// a step defers at most three children, and the builder only hands over hierarchies whose wide nodes are at most 42
+// levels deep (grandchildren nodes over a binary hierarchy of at most 62 levels, whose depth the Morton keys bound or
+// the build measures; nodes that open one level at a time only over hierarchies measured to be at most 42 deep).  A
+// stack that is full all the same loses the entry (no fault; checked on the builder's side, not here).
 // All active lanes share the direction signs `sgn` (bit a set = axis a negative), see slab_hit_fast.
 template <bool RESUME>
 __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySlab &slab, uint32_t sgn, F3 o, F3 d,

@@ -140,8 +140,8 @@ typedef struct DstAccelInfo {
     uint32_t n_internal;   /* internal nodes (n_surfels-1, 0 for a single surfel) */
     uint32_t root;         /* root reference (leaf bit set when n_surfels == 1) */
     uint32_t node_bytes, leaf_bytes;
-    float scene_lo[3], scene_hi[3]; /* bounds of the quad centroids used for the Morton grid */
-    float max_abs;         /* largest |coordinate| of any vertex */
+    float scene_lo[3], scene_hi[3]; /* bounds of the quad centroids used for the Morton grid, as of the last build */
+    float max_abs;         /* largest |coordinate| of any vertex, as of the last build or refit the device has finished */
     uint32_t builds, refits;
     uint32_t key_levels;   /* 1: the builds sort 30-bit Morton keys; 2: 60-bit keys in two levels, which a context goes
                               over to, for good, when a build finds more than three quarters of the surfels sharing

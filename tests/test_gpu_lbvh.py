@@ -235,6 +235,10 @@ def test_two_level_keys_are_given_up_when_the_hierarchy_gets_too_deep():
     far = _with_far_surfels(S.scene_cube(P=3000, seed=8), 2000.0)
     own.build_acceleration_structure(far["vertices"].cuda(), far["faces"].cuda(), True)
     assert own.optix_context.accel_info().key_levels == 1
+    # ... but not for ever: the sixteenth build after it tries the finer keys again (and keeps them for this scene)
+    for _ in range(15):
+        own.build_acceleration_structure(far["vertices"].cuda(), far["faces"].cuda(), True)
+    assert own.optix_context.accel_info().key_levels == 2
 
 
 def test_boundary_errors(tracer):
