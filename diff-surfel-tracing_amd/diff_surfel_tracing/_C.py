@@ -200,8 +200,9 @@ class OptiXStateWrapper:
         self.device = torch.cuda.current_device()
         self.num_surfels = 0
         self.record_blocks_per_wave = None  # sizing estimate for hit records: largest request seen, with headroom
-        self.record_max_bytes = 8 << 30     # no record larger than this is made (backward then re-traces)
-        self.record_pool_max_bytes = 16 << 30   # free storages kept for reuse, all together
+        self.record_max_bytes = 32 << 30    # no record larger than this is made (backward then re-traces); a 4K image
+                                            # of the 1M-surfel room scene needs 13 GB, of the card's 288
+        self.record_pool_max_bytes = 48 << 30   # free storages kept for reuse, all together
         self.records_skipped = 0            # forward calls that made no record because of the two limits above
         self.record_wanted = True           # set by the autograd wrapper for the call that follows
         self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
