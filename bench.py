@@ -208,6 +208,7 @@ def run_workload(key, steps, warmup, main, args):
     n_proc, n_con = counters.tolist()
 
     n_steps = len(frames) if frames else steps
+    handed_before = ctx.trace_info().tiles_handed_over
     fe = [(ev(), ev()) for _ in range(n_steps)]
     be = [(ev(), ev()) for _ in range(n_steps)]
     geo_ms = []
@@ -238,6 +239,8 @@ def run_workload(key, steps, warmup, main, args):
         torch.cuda.synchronize()
         trace_s = time.perf_counter() - t0
     ms_per_step = trace_s * 1e3 / n_steps
+    trace_info = ctx.trace_info()
+    handed = (trace_info.tiles_handed_over - handed_before) / n_steps
     fwd_ms = sum(a.elapsed_time(b) for a, b in fe) / n_steps   # kernel launch -> kernel end, on the launch stream
     bwd_ms = sum(a.elapsed_time(b) for a, b in be) / n_steps
     if frames and "means" in frames[-1]:
@@ -311,6 +314,9 @@ def run_workload(key, steps, warmup, main, args):
         "hits_evaluated_per_ray": round(n_proc / R, 3), "hits_composited_per_ray": round(n_con / R, 3),
         "hit_record": {"blocks_used": info.get("blocks"), "complete": info.get("complete"),
                        "allocated_bytes": info.get("record_bytes")},
+        # forward tiles whose packet walk ran into the step limit and were traced ray by ray by the second launch
+        "tile_handover": {"active": bool(trace_info.handover_active), "small_quads": trace_info.small_quads,
+                          "step_limit": trace_info.handover_steps, "tiles_per_forward": round(handed, 2)},
         "algorithmic_bytes": int(A_total),
         "reference_equivalent_hbm_frac": round(A_total / (ms_per_step * 1e-3) / (HBM_PEAK_GBS * 1e9), 5),
         "roofline_kernels": per_kernel,

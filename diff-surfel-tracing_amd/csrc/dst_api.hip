@@ -61,10 +61,24 @@ dst_ctx *dst_create(void) {
         return nullptr;
     }
     if (const char *h = std::getenv("DST_HIERARCHY")) ctx->use_ploc = std::strcmp(h, "morton") != 0;
+    if (const char *h = std::getenv("DST_HANDOVER_STEPS")) {
+        const unsigned long v = std::strtoul(h, nullptr, 10);
+        if (v != 0ul) ctx->handover_steps = (uint32_t)std::min<unsigned long>(v, 1ul << 30);
+    }
+    if (const char *h = std::getenv("DST_HANDOVER"))
+        ctx->handover_mode = std::strcmp(h, "off") == 0 ? DST_HANDOVER_OFF
+                                                        : (std::strcmp(h, "always") == 0 ? DST_HANDOVER_ALWAYS : DST_HANDOVER_AUTO);
     if (dst_static_scratch_init(ctx) != DST_OK) {   // once per device, with that device current
         delete ctx;
         return nullptr;
     }
+    const size_t bytes = kDstHandoverOffset + sizeof(uint32_t) * (kDstHandoverHeader + kDstHandoverCap);
+    if (hipMalloc((void **)&ctx->bounds, bytes) != hipSuccess || hipMemset(ctx->bounds, 0, bytes) != hipSuccess ||
+        hipDeviceSynchronize() != hipSuccess) {
+        dst_destroy(ctx);
+        return nullptr;
+    }
+    ctx->handover = dst_handover_list(ctx->bounds);
     return ctx;
 }
 
@@ -165,6 +179,30 @@ int dst_trace_backward(dst_ctx *ctx, const DstParams *p, void *stream) {
     if (p->shs && !p->dL_dshs) return dst_fail(ctx, DST_E_INVALID, "dL_dshs missing");
     if (p->others_precomp && !p->dL_dothers) return dst_fail(ctx, DST_E_INVALID, "dL_dothers missing");
     return dst_launch_trace(ctx, *p, true, (hipStream_t)stream);
+}
+
+int dst_trace_info(dst_ctx *ctx, DstTraceInfo *info) {
+    if (!ctx || !info) return DST_E_INVALID;
+    uint32_t words[kDstHandoverHeader] = {};
+    DST_HIP(ctx, hipDeviceSynchronize());
+    DST_HIP(ctx, hipMemcpy(words, ctx->handover, sizeof(words), hipMemcpyDeviceToHost));
+    info->handover_mode = (uint32_t)ctx->handover_mode;
+    info->handover_steps = ctx->handover_steps;
+    info->handover_capacity = kDstHandoverCap;
+    info->small_quads = ctx->small_quads;
+    info->handover_active = dst_handover_active(ctx) ? 1u : 0u;
+    info->reserved = 0u;
+    info->tiles_handed_over = words[2];
+    return DST_OK;
+}
+
+int dst_set_handover(dst_ctx *ctx, int mode, uint32_t steps) {
+    if (!ctx) return DST_E_INVALID;
+    if (mode != DST_HANDOVER_OFF && mode != DST_HANDOVER_AUTO && mode != DST_HANDOVER_ALWAYS)
+        return dst_fail(ctx, DST_E_INVALID, "hand-over mode must be DST_HANDOVER_OFF, _AUTO or _ALWAYS");
+    ctx->handover_mode = mode;
+    if (steps != 0u) ctx->handover_steps = std::min<uint32_t>(steps, 1u << 30);
+    return DST_OK;
 }
 
 int dst_pack_sh_half(const float *shs, uint16_t *out, uint64_t n_values, void *stream) {

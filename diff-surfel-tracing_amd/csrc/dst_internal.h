@@ -70,7 +70,13 @@ struct DstBounds {          // device-resident reduction targets, order-preservi
     uint32_t max_depth;     // nodes above the deepest leaf (builds with two-level keys only)
     uint32_t scale;         // raw bits of a float: size of the scene's bulk (set by a build, kept by refits); what ray
                             // origins are compared with (packets, ray keys) - not a bound on anything
+    uint32_t small_quads;   // quads with edges below kDstSmallQuad of that size, counted by a build
 };
+// Quads this much smaller than the scene are smaller than a pixel at usual resolutions (a 1080p pixel at half the
+// scene's size away is about 5e-4 of it wide); a context whose last build counted kDstSmallQuadsMin of them traces
+// with the kernels that can hand a tile over (trace.hip), the others with kernels that do not carry that code.
+constexpr float kDstSmallQuad = 1.0f / 2048.0f;
+constexpr uint32_t kDstSmallQuadsMin = 2048;
 
 // Device-side view of the acceleration structure handed to the trace kernels.
 struct DstAccelView {
@@ -82,6 +88,20 @@ struct DstAccelView {
     uint32_t root;
     uint32_t n_leaves;
 };
+
+// Tile hand-over list of the forward trace (layout: trace.hip).  Steps: walks of the benchmark scenes take a few
+// hundred; DST_HANDOVER_STEPS in the environment of dst_create sets another limit.
+constexpr uint32_t kDstHandoverHeader = 4, kDstHandoverCap = 8192, kDstHandoverSteps = 2048;
+// The list shares its allocation with the bounds (made by dst_create).
+constexpr size_t kDstHandoverOffset = 64;   // bytes from the bounds to the list
+static_assert(sizeof(DstBounds) <= kDstHandoverOffset, "the hand-over list starts behind the bounds");
+__host__ __device__ static inline uint32_t *dst_handover_list(const DstBounds *bounds) {
+    return reinterpret_cast<uint32_t *>(reinterpret_cast<uintptr_t>(bounds) + kDstHandoverOffset);
+}
+
+struct dst_ctx;
+// Whether the context's next forward trace uses the kernels that can hand tiles over.
+static inline bool dst_handover_active(const dst_ctx *ctx);
 
 struct dst_ctx {
     int device = 0;
@@ -121,11 +141,22 @@ struct dst_ctx {
     uint32_t ray_capacity = 0;
     uint32_t *block_order = nullptr;   // dispatch order of a replaying backward trace (longest blocks first), grow-only
     uint32_t block_order_capacity = 0;
-    DstBounds *bounds = nullptr;       // device
+    // forward traces: tiles whose packet walk ran long, handed over to waves that walk every ray on its own (trace.hip)
+    uint32_t *handover = nullptr;      // device, behind `bounds`: kDstHandoverHeader words + kDstHandoverCap entries, zeroed at creation
+    uint32_t handover_steps = kDstHandoverSteps;   // limit of a tile's first walk
+    int handover_mode = DST_HANDOVER_AUTO;         // auto: only for scenes with many small quads
+    uint32_t small_quads = 0;          // as counted by the last build
+    uint32_t handover_parity = 0;      // which of the list's two counters the next trace counts in
+    DstBounds *bounds = nullptr;       // device (allocated by dst_create together with the hand-over list)
     DstBounds *bounds_host = nullptr;  // pinned host copy
     void *core_box = nullptr;          // device: the box the two-level Morton keys are laid over (lbvh.hip)
     float scene_lo[3] = {0, 0, 0}, scene_hi[3] = {0, 0, 0}, max_abs = 0;
 };
+
+static inline bool dst_handover_active(const dst_ctx *ctx) {
+    if (ctx->handover_mode == DST_HANDOVER_OFF || ctx->handover_steps == 0u || ctx->handover == nullptr) return false;
+    return ctx->handover_mode == DST_HANDOVER_ALWAYS || ctx->small_quads >= kDstSmallQuadsMin;
+}
 
 // Where a traversal starts: the wide node of the binary root, or one leaf group when the scene is that small.
 static inline uint32_t dst_root_ref(uint32_t n_leaves) {

@@ -46,6 +46,7 @@ __global__ void k_init_bounds(DstBounds *b) {
         b->bad_topology = 0u;
         b->equal_keys = 0u;
         b->max_depth = 0u;
+        b->small_quads = 0u;
     }
 }
 
@@ -769,15 +770,27 @@ __global__ void k_fit_ranges(DstNode *nodes, RangeBoxes rb, uint32_t n_blocks, u
 // Leaf records in Morton order (also the whole of a refit's geometry update).
 __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
                             const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
-                            DstLeafPre *__restrict__ pre, RangeBoxes rb, DstBounds *__restrict__ bounds, uint32_t n) {
+                            DstLeafPre *__restrict__ pre, RangeBoxes rb, DstBounds *__restrict__ bounds,
+                            DstBounds *__restrict__ count_small, uint32_t n) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     const bool valid = i < n;   // every lane stays for the wave-wide scans of the boxes
     float c[4][3] = {};
     float mabs = 0.f;
+    bool small = false;
     if (valid) {
         const uint32_t g = sorted_ids[i];
         load_corners(vertices, quad_ids[g], g, c);
         write_leaf(c, g, i, leaves, pre);
+        if (count_small != nullptr) {   // a build: quads far smaller than the scene (DstBounds::small_quads)
+            float ab = 0.f, ac = 0.f;
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                ab += (c[1][a] - c[0][a]) * (c[1][a] - c[0][a]);
+                ac += (c[2][a] - c[0][a]) * (c[2][a] - c[0][a]);
+            }
+            const float lim = __uint_as_float(count_small->scale) * kDstSmallQuad;
+            small = fmaxf(ab, ac) < lim * lim;
+        }
 #pragma unroll
         for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -785,6 +798,10 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
     }
     if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
     if (bounds != nullptr) block_max_abs(mabs, bounds);   // a refit: the coordinate bound of the moved quads
+    if (count_small != nullptr) {
+        const unsigned long long m = __ballot(small);
+        if ((threadIdx.x & (DST_WAVE - 1)) == 0 && m != 0ull) atomicAdd(&count_small->small_quads, (uint32_t)__popcll(m));
+    }
 }
 
 // The same for a refit straight from the surfel parameters: the four corners of surfel g are
@@ -1297,7 +1314,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     }
     if (surfels == nullptr)
         hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0],
-                           ctx->leaves, ctx->pre, rb, rebuild ? nullptr : ctx->bounds, n);
+                           ctx->leaves, ctx->pre, rb, rebuild ? nullptr : ctx->bounds, rebuild ? ctx->bounds : nullptr, n);
     if (by_ranges) {
         const uint32_t n_blocks = (n + kRangeBlock - 1) / kRangeBlock;
         for (int level = 1; (2u << (level - 1)) <= n_blocks; ++level)
@@ -1334,6 +1351,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
             ctx->scene_hi[a] = ord2f(ctx->bounds_host->hi[a]);
         }
         std::memcpy(&ctx->max_abs, &ctx->bounds_host->max_abs, 4);
+        ctx->small_quads = ctx->bounds_host->small_quads;
         if (ctx->fine_keys && ctx->bounds_host->max_depth > kMaxDepth) {
             // deeper than the walks' stacks are sized for (nested clusters at every scale): one-level keys, for good
             ctx->fine_keys = false;

@@ -502,6 +502,8 @@ struct WalkList {
     lds_u32 in, out;   // kListCap words each (LDS of this wave)
     uint32_t n_in;     // items in `in`, or kListFresh
     bool record;       // write `out` (false: plain walks from the root)
+    uint32_t limit;    // steps this walk may take at most (0: as many as the hierarchy can need)
+    bool spent;        // set by a walk that ran into its limit: its buffer is not to be used
 };
 
 // One traversal for the whole wave: every active lane ends with its own 16 nearest hits (t relative
@@ -512,7 +514,7 @@ struct WalkList {
 // the build measures; nodes that open one level at a time only over hierarchies measured to be at most 42 deep).  A
 // stack that is full all the same loses the entry (no fault; checked on the builder's side, not here).
 // All active lanes share the direction signs `sgn` (bit a set = axis a negative), see slab_hit_fast.
-template <bool RESUME>
+template <bool RESUME, bool HAND>
 __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySlab &slab, uint32_t sgn, F3 o, F3 d,
                                             bool active, int rep, KBuf &buf, uint32_t &cnt, WalkList &wl
 #ifdef DST_STATS
@@ -543,6 +545,9 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
     // copies of the buffer's 32 registers and moved them back and forth at every leaf group).
     constexpr uint32_t kEnd = 0xFFFFFFFFu;   // not a reference: leaf bit set, impossible position
     uint32_t budget = 2u * acc.n_leaves + 8u;
+    if constexpr (RESUME && HAND) {
+        if (wl.limit != 0u) budget = min(budget, wl.limit);
+    }
     // The work lists are read and written a page of 64 items at a time: lane k of a page register holds item k.
     uint32_t in_page = 0u, out_page = 0u, in_pos = 0u, n_out = 0u;
     const uint32_t n_in = (RESUME && wl.n_in != kListFresh) ? wl.n_in : 0u;
@@ -654,6 +659,9 @@ __device__ __forceinline__ void packet_walk(const DstAccelView &acc, const RaySl
         ref = pop();
     }
     if (RESUME) {
+        if constexpr (HAND) {
+            if (wl.limit != 0u && budget == 0u) wl.spent = true;
+        }
         if (recording) {
             // a walk that stopped early (budget, damaged structure) or a list that overflowed leaves no list
             const bool whole = n_out <= kListCap && budget != 0u && ref == kEnd;
@@ -846,7 +854,7 @@ __device__ __forceinline__ bool rays_run_together(F3 o, F3 d, bool active, float
     return wave_ballot(apart) == 0ull;
 }
 
-template <bool MIXED, bool SHELF, bool RESUME>
+template <bool MIXED, bool SHELF, bool RESUME, bool HAND>
 __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_abs, F3 o, F3 d, bool active, KBuf &buf,
                                            uint32_t &cnt, bool as_packet, WalkList &wl, uint32_t *shelf
 #ifdef DST_STATS
@@ -882,7 +890,7 @@ __device__ __forceinline__ void packet_knn(const DstAccelView &acc, float max_ab
         const uint32_t sgn = __builtin_amdgcn_readlane(my_sgn, rep);
         const bool mine = active && my_sgn == sgn;
         todo &= ~wave_ballot(mine);
-        packet_walk<RESUME>(acc, slab, sgn, o, d, mine, rep, buf, cnt, wl WSP);
+        packet_walk<RESUME, HAND>(acc, slab, sgn, o, d, mine, rep, buf, cnt, wl WSP);
     }
 }
 
@@ -1504,12 +1512,17 @@ __device__ __forceinline__ void table_clear_keys(uint32_t *keys) {
 
 // One bounce: chunked 16-nearest traversal + front-to-back compositing (reference forward.cu:136-315),
 // and for BWD the per-hit gradients of the re-trace (reference backward.cu:332-655).
-template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
-__device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
+// `first_walk` (forward): 0, or the number of steps the packet walk of the bounce's first chunk may take before the
+// wave gives its tile up (returns true, nothing written yet: see the tile hand-over in trace_body), or kWalkPerLane:
+// every ray of the wave walks on its own whatever the rays look like (the waves that take such tiles over).
+// HAND: kernels without the hand-over do not contain its code at all (first_walk is ignored).
+constexpr uint32_t kWalkPerLane = 0xFFFFFFFFu;
+template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET, bool HAND>
+__device__ __forceinline__ bool walk_bounce(const DstParams &p, const DstAccelView &acc, float max_abs, bool lane_on,
                                             F3 ro, F3 rd, float min_depth, BounceAcc<AUXM> &run,
                                             const BounceIn<AUXM> &in, F3 &g_ro, F3 &g_rd, uint32_t &n_proc,
                                             uint32_t &n_con, uint32_t *tab_keys, float *tab_rows, float *stage,
-                                            const RecView &rv, int bounce, F3 &dist_acc
+                                            const RecView &rv, int bounce, F3 &dist_acc, uint32_t first_walk
 #ifdef DST_STATS
                                             , WaveStats &ws
 #endif
@@ -1527,7 +1540,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     LastShHit last_sh = {0, f3(0, 0, 0), false};
     STAT(last_sh.t_alg = 0; last_sh.t_sh = 0;)
     // kernels built without the per-lane walk (MIXED false) take every wave as a packet
-    const bool as_packet = (!MIXED || (REC && BWD)) ? true : rays_run_together(ro, rd, lane_on, max_abs);
+    const bool as_packet = (!MIXED || (REC && BWD)) ? true
+                                                    : (HAND && first_walk == kWalkPerLane ? false : rays_run_together(ro, rd, lane_on, max_abs));
     // Forward: the walks of a bounce's later chunks resume from the list the walk before left (the backward
     // re-trace has its LDS taken by the gradient table and walks from the root).
     constexpr bool RESUME = !BWD;
@@ -1544,6 +1558,8 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     wl.out = wl.in + (RESUME ? kListCap : 0);
     wl.n_in = kListFresh;
     wl.record = false;
+    wl.limit = (HAND && first_walk != kWalkPerLane) ? first_walk : 0u;
+    wl.spent = false;
     uint32_t rec_pos = (REC && BWD) ? (rv.dir[bounce] & kRecDirBlockMask) : 0xFFFFFFFFu;   // replay: next block + 1; record: previous block
     uint32_t rec_chunks = 0u;   // forward with a record: chunks stored for this bounce
     for (;;) {
@@ -1572,7 +1588,11 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
             }
         } else {
             kbuf_reset(buf);
-            packet_knn<MIXED, SHELF, RESUME>(acc, max_abs, ot, rd, live, buf, cnt, as_packet, wl, wave_lds WSP);
+            packet_knn<MIXED, SHELF, RESUME, HAND>(acc, max_abs, ot, rd, live, buf, cnt, as_packet, wl, wave_lds WSP);
+            if constexpr (HAND) {
+                if (wl.spent) return true;   // only a bounce's first walk has a limit: nothing has been written yet
+                wl.limit = 0u;
+            }
             if (REC && !BWD) {
                 rec_colours = rec_store(rv, bounce, rec_pos, buf, cnt);
                 rec_chunks += rec_colours != nullptr ? 1u : 0u;
@@ -1786,6 +1806,7 @@ __device__ __forceinline__ void walk_bounce(const DstParams &p, const DstAccelVi
     if (BWD && p.colors_precomp == nullptr && last_sh.any)
         g_rd = sh_direction_gradient(p.D, ShF32{p.shs + (size_t)last_sh.g * p.M * 3}, rd, last_sh.gc);
     run.T = Tp;
+    return false;
 }
 
 __device__ __forceinline__ F3 dnormvdv(F3 v, F3 dv) {
@@ -1875,11 +1896,23 @@ __global__ __launch_bounds__(1024) void k_block_order(const uint32_t *__restrict
     }
 }
 
-template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET>
+// Tile hand-over (forward).  A packet walk visits what any of its 64 rays needs, one dependent fetch after the other.
+// Over geometry much finer than the ray spacing (a dense cloud of surfels far smaller than a pixel) that is the whole
+// content of the tile's frustum, wanted by one ray at best, and a single wave walks for milliseconds while the chip
+// idles.  So the first walk of a tile may take `hand_arg` steps (bits 0..30) and no more: a wave that runs into that
+// limit has written nothing yet, puts its tile on the context's list and leaves, and a second, small launch right
+// behind (kernels with the per-lane walk, hand_arg steps = 0: the takers) traces the listed tiles with every ray
+// walking on its own - the same buffer content, so the same results bit for bit.  List: word 0 / 1 = tiles listed by
+// the trace of even / odd parity (hand_arg bit 31; a trace's takers clear the word the next trace will count in),
+// word 2 = tiles handed over since the context was made, entries ((by * btiles_x + bx) * 4 + wave) from word 4.  A
+// wave that finds the list full starts again without a limit.
+constexpr uint32_t kHandHeader = kDstHandoverHeader, kHandCap = kDstHandoverCap, kHandStepsMask = 0x7FFFFFFFu;
+template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET, bool HAND>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x,
                                            const uint32_t *__restrict__ ray_order, uint32_t strip_width,
-                                           const uint32_t *__restrict__ block_order) {
+                                           const uint32_t *__restrict__ block_order, uint32_t *handover,
+                                           uint32_t hand_arg) {
     // a block = 2x2 wave tiles (16x16 pixels for the usual 8x8 tile): neighbouring rays share surfels, which
     // is what the block's gradient table and the caches live on
     constexpr int kTableRows = RowLayout<AUXM>::rows;
@@ -1932,7 +1965,23 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     // narrower; its blocks are spread over all XCDs like the others.  The launcher chooses the width (launch()).
     if (BWD && block_order != nullptr) bid = block_order[bid];   // replay: the longest blocks first (k_block_order)
     uint32_t bx, by;
+    static_assert(!HAND || (!BWD && kFwdWavesPerBlock == 1), "tiles are handed over by forward kernels of one wave per workgroup");
+    const bool taker = HAND && MIXED && handover != nullptr && (hand_arg & kHandStepsMask) == 0u;
     block_of_position(bid, btiles_x, (tiles_y + 1u) / 2u, strip_width, th_log2 != 0, bx, by);
+    if constexpr (HAND) {
+        if (taker) {   // the tile comes from the list, not from the workgroup's number
+            const uint32_t par = hand_arg >> 31, n = min(handover[par], gridDim.x);
+            if (blockIdx.x == 0u && threadIdx.x == 0u) {
+                handover[par ^ 1u] = 0u;
+                handover[2] += n;
+            }
+            if (blockIdx.x >= n) return;
+            const uint32_t id = handover[kHandHeader + blockIdx.x];
+            wv = id & 3u;
+            bx = (id >> 2) % btiles_x;
+            by = (id >> 2) / btiles_x;
+        }
+    }
     const bool flat = th_log2 == 0;   // a ray list: tiles of 1x64 rays, a block = four consecutive tiles
     if (flat ? by >= 1u : 2u * by >= tiles_y) return;   // padding of the forward grid (whole blocks)
     RecView rv = {nullptr, nullptr, nullptr, 0u};
@@ -1977,10 +2026,23 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         F3 ot = ray_o, dt = ray_d;
         float s_prod = 1.0f;
         bool on = inside;
+        uint32_t first_walk = (HAND && handover != nullptr) ? (hand_arg & kHandStepsMask) : 0u;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             F3 dist_acc = f3(0, 0, 0);
-            walk_bounce<false, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, WET ? wet_keys : nullptr, WET ? wet_vals : nullptr, nullptr, rv, i, dist_acc WS_ARG);
+            const bool gave_up = walk_bounce<false, AUXM, REC, MIXED, DET, HAND>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, WET ? wet_keys : nullptr, WET ? wet_vals : nullptr, nullptr, rv, i, dist_acc, taker ? kWalkPerLane : (i == 0 ? first_walk : 0u) WS_ARG);
+            if constexpr (HAND) if (gave_up) {   // (bounce 0, before anything was written; no else below)
+                uint32_t slot = 0u;
+                if (lane == 0u) slot = atomicAdd(&handover[hand_arg >> 31], 1u);
+                slot = __builtin_amdgcn_readfirstlane(slot);
+                if (slot < kHandCap) {
+                    if (lane == 0u) handover[kHandHeader + slot] = ((by * btiles_x + bx) << 2) | wv;
+                    return;
+                }
+                first_walk = 0u;   // the list is full: this wave keeps its tile
+                --i;
+                continue;
+            }
             if (on) {
                 run.C[0] += run.T * p.background[0];
                 run.C[1] += run.T * p.background[1];
@@ -2131,7 +2193,7 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
             }
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             F3 no_dist = f3(0, 0, 0);
-            walk_bounce<true, AUXM, REC, MIXED, DET>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i, no_dist WS_ARG);
+            (void)walk_bounce<true, AUXM, REC, MIXED, DET, false>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, tab_keys, tab_rows, s_stage + wv * kStageWords, rv, i, no_dist, 0u WS_ARG);
         }
 #ifdef DST_STATS   // development build only: counters must then hold 11 entries
         if (p.counters != nullptr && lane == 0) {
@@ -2168,15 +2230,25 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
 template <int AUXM, bool REC, bool MIXED, bool EXTRAS>
 __global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
 void k_trace_fwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
-                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width) {
-    trace_body<false, AUXM, REC, MIXED, EXTRAS>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, nullptr);
+                 uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width, uint32_t *handover,
+                 uint32_t hand_arg) {
+    trace_body<false, AUXM, REC, MIXED, EXTRAS, kFwdWavesPerBlock == 1>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, nullptr, handover, hand_arg);
+}
+// The forward kernel of image grids at depth 0 without the tile hand-over: what scenes without many small quads are
+// traced with (the hand-over's few extra live values cost the walk 1 to 4 % of its time through the register
+// allocation, whether a tile is ever handed over or not).
+template <int AUXM, bool REC>
+__global__ __launch_bounds__(kFwdWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_FWD_WAVES, DST_FWD_WAVES)))
+void k_trace_fwd_plain(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
+                       uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width) {
+    trace_body<false, AUXM, REC, false, false, false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, nullptr, nullptr, 0u);
 }
 template <int AUXM, bool REC, bool MIXED, bool DET>
 __global__ __launch_bounds__(kWavesPerBlock *DST_WAVE) __attribute__((amdgpu_waves_per_eu(DST_BWD_WAVES, DST_BWD_WAVES)))
 void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_log2, uint32_t tiles_x,
                  uint32_t tiles_y, uint32_t btiles_x, const uint32_t *ray_order, uint32_t strip_width,
                  const uint32_t *block_order) {
-    trace_body<true, AUXM, REC, MIXED, DET>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, block_order);
+    trace_body<true, AUXM, REC, MIXED, DET, false>(p, acc, tw_log2, th_log2, tiles_x, tiles_y, btiles_x, ray_order, strip_width, block_order, nullptr, 0u);
 }
 
 // Closing kernels of the deterministic mode: fixed point -> fp32, added to the caller's (zero-filled) tensors.
@@ -2288,14 +2360,17 @@ TileGrid tile_grid(int H, int W) {
     return t;
 }
 
+// `handover` / `hand_arg`: see trace_body (forward only; hand_arg steps = 0 launches the takers of the listed tiles).
 template <bool BWD, bool REC>
 void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, const uint32_t *ray_order, hipStream_t stream,
-            const uint32_t *block_order = nullptr) {
+            const uint32_t *block_order = nullptr, uint32_t *handover = nullptr, uint32_t hand_arg = 0u) {
     const uint32_t n_blocks = t.btiles_x * t.btiles_y;
     dim3 grid(n_blocks), block(kWavesPerBlock * DST_WAVE);
+    const bool takers = !BWD && handover != nullptr && (hand_arg & kHandStepsMask) == 0u;
     if (!BWD && kFwdWavesPerBlock == 1) {
         grid = dim3((n_blocks + 7u) / 8u * 32u);
         block = dim3(DST_WAVE);
+        if (takers) grid = dim3(std::min<uint32_t>(n_blocks * (uint32_t)kWavesPerBlock, kHandCap));
     }
     // The per-lane walk is built into the kernels used where waves of unrelated rays are to be expected:
     // reflection bounces and ray lists (thin grids).  Image-shaped grids traced to depth 0 get the pure packet kernels.
@@ -2306,7 +2381,7 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
     // The backward trace gains 1 to 3 % from strips of 8 on every grid measured.
     uint32_t strip = 0u;
     if (t.th_log2 != 0) strip = BWD ? (uint32_t)DST_STRIP_BWD : (n_blocks >= kStripMinBlocks ? (uint32_t)DST_STRIP_FWD : 0u);
-    const bool mixed = p.max_trace_depth > 0 || t.th_log2 < 3;
+    const bool mixed = takers || p.max_trace_depth > 0 || t.th_log2 < 3;
     const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
 #define DST_LAUNCH_M(AUX, MIXED)                                                                                   \
     do {                                                                                                           \
@@ -2316,12 +2391,15 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
         else if (BWD)                                                                                              \
             hipLaunchKernelGGL((k_trace_bwd<AUX, REC, (MIXED) && !REC, false>), grid, block, 0, stream, p, acc,     \
                                t.tw_log2, t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip, block_order);    \
+        else if (!(MIXED) && p.flags == 0u && handover == nullptr)                                                 \
+            hipLaunchKernelGGL((k_trace_fwd_plain<AUX, REC>), grid, block, 0, stream, p, acc, t.tw_log2,           \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                            \
         else if (p.flags != 0u)                                                                                    \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, true>), grid, block, 0, stream, p, acc, t.tw_log2,    \
-                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                            \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip, handover, hand_arg);        \
         else                                                                                                       \
             hipLaunchKernelGGL((k_trace_fwd<AUX, REC, MIXED, false>), grid, block, 0, stream, p, acc, t.tw_log2,   \
-                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip);                            \
+                               t.th_log2, t.tiles_x, t.tiles_y, t.btiles_x, ray_order, strip, handover, hand_arg);        \
     } while (0)
 #define DST_LAUNCH(AUX)                                                                                            \
     do {                                                                                                           \
@@ -2441,8 +2519,16 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
             else hipLaunchKernelGGL(k_finish_grad_rows<8>, grid, block, 0, stream, p);
         }
     } else {
-        if (rec) launch<false, true>(p, acc, t, ray_order, stream);
-        else launch<false, false>(p, acc, t, ray_order, stream);
+        // the second launch of each pair traces the tiles the first one handed over (usually none: it leaves at once)
+        uint32_t *const list = (kFwdWavesPerBlock == 1 && dst_handover_active(ctx)) ? ctx->handover : nullptr;
+        const uint32_t parity = (uint32_t)(ctx->handover_parity & 1u) << 31;
+        const uint32_t steps = std::min<uint32_t>(ctx->handover_steps, kHandStepsMask);
+        for (int pass = 0; pass < (list != nullptr ? 2 : 1); ++pass) {
+            const uint32_t arg = parity | (pass == 0 ? steps : 0u);
+            if (rec) launch<false, true>(p, acc, t, ray_order, stream, nullptr, list, arg);
+            else launch<false, false>(p, acc, t, ray_order, stream, nullptr, list, arg);
+        }
+        if (list != nullptr) ctx->handover_parity ^= 1u;
         if (det && p.training && p.a_weights != nullptr)
             hipLaunchKernelGGL(k_det_finish_weights, dim3(1024), dim3(256), 0, stream, p);
     }

@@ -49,10 +49,19 @@ class DstAccelInfo(C.Structure):
                 ("key_levels", C.c_uint32), ("agglomerated", C.c_uint32), ("depth", C.c_uint32)]
 
 
+class DstTraceInfo(C.Structure):
+    _fields_ = [("handover_mode", C.c_uint32), ("handover_steps", C.c_uint32), ("handover_capacity", C.c_uint32),
+                ("small_quads", C.c_uint32), ("handover_active", C.c_uint32), ("reserved", C.c_uint32),
+                ("tiles_handed_over", C.c_uint64)]
+
+
+HANDOVER_OFF, HANDOVER_AUTO, HANDOVER_ALWAYS = 0, 1, 2
+
+
 EXPORTS = ("dst_create", "dst_destroy", "dst_build_accel", "dst_trace_forward", "dst_trace_backward",
            "dst_last_error", "dst_accel_info", "dst_accel_download", "dst_version", "dst_sizeof_params",
            "dst_hit_record_layout", "dst_refit_accel_static", "dst_refit_from_surfels",
-           "dst_det_workspace_words", "dst_pack_sh_half")
+           "dst_det_workspace_words", "dst_pack_sh_half", "dst_trace_info", "dst_set_handover")
 
 _lib = None
 
@@ -80,6 +89,8 @@ def load_library():
     L.dst_last_error.argtypes = [C.c_void_p]
     L.dst_accel_info.argtypes = [C.c_void_p, C.POINTER(DstAccelInfo)]
     L.dst_accel_download.argtypes = [C.c_void_p] * 7
+    L.dst_trace_info.argtypes = [C.c_void_p, C.POINTER(DstTraceInfo)]
+    L.dst_set_handover.argtypes = [C.c_void_p, C.c_int, C.c_uint32]
     L.dst_det_workspace_words.restype = C.c_uint64
     L.dst_det_workspace_words.argtypes = [C.c_int32, C.c_int32, C.c_int]
     L.dst_pack_sh_half.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
@@ -301,6 +312,18 @@ class OptiXStateWrapper:
         info = DstAccelInfo()
         _check(self, load_library().dst_accel_info(self.handle, C.byref(info)))
         return info
+
+    def trace_info(self):
+        """Tile hand-over of the forward trace (include/dst_api.h): mode, step limit, list capacity, the small quads the
+        last build counted, whether the next forward trace can hand over, tiles handed over so far.  Waits."""
+        info = DstTraceInfo()
+        _check(self, load_library().dst_trace_info(self.handle, C.byref(info)))
+        return info
+
+    def set_handover(self, mode, steps=0):
+        """HANDOVER_OFF / HANDOVER_AUTO (only for scenes with many quads far smaller than the scene) / HANDOVER_ALWAYS;
+        `steps`: what a tile's first packet walk may take before its rays are walked one by one (0: unchanged)."""
+        _check(self, load_library().dst_set_handover(self.handle, int(mode), int(steps)))
 
     def __del__(self):
         h, self.handle = getattr(self, "handle", None), None

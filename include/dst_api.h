@@ -215,6 +215,32 @@ int dst_accel_info(dst_ctx *ctx, DstAccelInfo *info);
 int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_parent, uint32_t *leaf_parent,
                        uint32_t *sorted_keys, void *stream);
 
+/* Tile hand-over of the forward trace (no counterpart in the reference, whose rays are traversed one by one by the
+ * hardware: optix_tracer/forward.cu:318).  The trace kernels walk the BVH once for the 64 rays of an 8x8 pixel tile.
+ * Over geometry much finer than the ray spacing (a dense cloud of surfels far smaller than a pixel) that walk visits
+ * everything inside the tile's frustum for the sake of one ray at a time, and one wave runs for milliseconds.  A tile
+ * whose first walk takes more than `handover_steps` steps (nodes and leaf groups; default 2048, a few hundred on
+ * ordinary scenes) is therefore put on a list and traced by a second launch in which every ray walks on its own: same
+ * results bit for bit.  At most `handover_capacity` tiles per call are handed over; further ones are traced the usual
+ * way.  The kernels that can hand over are 1 to 4 % slower than those that cannot, so by default (DST_HANDOVER_AUTO)
+ * a context uses them only while its last build counted at least 2048 quads with edges below 1/2048 of the scene's
+ * size (`small_quads`; refits do not recount); DST_HANDOVER_ALWAYS and DST_HANDOVER_OFF decide regardless of the
+ * scene.  dst_set_handover: steps = 0 keeps the current limit.  DST_HANDOVER=off|auto|always and DST_HANDOVER_STEPS=n
+ * in the environment of dst_create set the initial values.  dst_trace_info waits for the device; tiles_handed_over
+ * counts since the context was created (a 32-bit count). */
+#define DST_HANDOVER_OFF 0
+#define DST_HANDOVER_AUTO 1
+#define DST_HANDOVER_ALWAYS 2
+typedef struct DstTraceInfo {
+    uint32_t handover_mode, handover_steps, handover_capacity;
+    uint32_t small_quads;        /* as counted by the last build */
+    uint32_t handover_active;    /* 1: the next forward trace uses the kernels that can hand tiles over */
+    uint32_t reserved;
+    uint64_t tiles_handed_over;
+} DstTraceInfo;
+int dst_trace_info(dst_ctx *ctx, DstTraceInfo *info);
+int dst_set_handover(dst_ctx *ctx, int mode, uint32_t steps);
+
 /* Size in 8-byte words of a hit record with room for `blocks` chunk blocks, for an (H,W) ray grid traced with
  * `mtd_alloc`.  Also returns the words of the header the caller must zero-fill, and the number of waves the
  * grid is traced with (a forward trace at depth 0 asks for about 3-6 blocks per wave). */
