@@ -38,16 +38,21 @@ struct alignas(128) DstWideNode {
     uint32_t pad[3];
 };
 
-// Leaf = one surfel quad in Morton order: corners A,B,C,D (triangles ABC and BCD), the two plane normals
-// n0 = (B-A)x(C-A), n1 = (C-B)x(D-B) as the hit test defines them, and the surfel id.  80 bytes, fetched
-// once per wave.
+// Leaf = one surfel quad in leaf order (triangles ABC and BCD), as the hit test wants it: corner A, the edge vectors
+// AB = B-A, AC = C-A, AD = D-A (fp32 differences of the corners), the plane normals n0 = AB x AC, n1 = (C-B)x(D-B),
+// n2 = AC x AD, c1 = n1.AB (crosses and dots in the fused form the test is defined with), and the surfel id.
+// 96 bytes, fetched once per wave.  The first 64 bytes hold what cannot be derived (n1 is formed from the corners B, C,
+// D, which A + AB and so on need not give back); n0, n2 and c1 follow from them by the same fp32 operations, so the
+// per-lane walk, whose every lane fetches its own quads, reads 64 bytes and computes them.
 struct alignas(16) DstLeaf {
-    float A[3], B[3], C[3], D[3];
-    float n0[3], n1[3];
+    float A[3], AB[3], AC[3], AD[3];
+    float n1[3];
     uint32_t g;
+    float n0[3], n2[3];
+    float c1;
     uint32_t pad;
 };
-static_assert(sizeof(DstLeaf) == 80, "leaf records are 20 dwords");
+static_assert(sizeof(DstLeaf) == 96, "leaf records are 24 dwords");
 
 // Cheap conservative stand-in for the exact ray/quad test, one per leaf (same order): the quad as a parallelogram
 // on its mean plane.  A ray whose hit point on that plane has |s|, |r| beyond `lim0` (plus a margin for rounding)

@@ -579,30 +579,36 @@ __device__ __forceinline__ void write_leaf(const float (&c)[4][3], uint32_t g, u
         out[1] = __builtin_fmaf(x[2], y[0], -(x[0] * y[2]));
         out[2] = __builtin_fmaf(x[0], y[1], -(x[1] * y[0]));
     };
-    float e1[3], e2[3], f1[3], f2[3], n0[3], n1[3];
+    float e1[3], e2[3], e3[3], f1[3], f2[3], n0[3], n1[3], n2[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
         e1[a] = c[1][a] - c[0][a];   // B - A
         e2[a] = c[2][a] - c[0][a];   // C - A
+        e3[a] = c[3][a] - c[0][a];   // D - A
         f1[a] = c[2][a] - c[1][a];   // C - B
         f2[a] = c[3][a] - c[1][a];   // D - B
     }
     cross_f(e1, e2, n0);
     cross_f(f1, f2, n1);
-    float out[20];
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-        for (int a = 0; a < 3; ++a) out[3 * k + a] = c[k][a];
+    cross_f(e2, e3, n2);
+    const float c1 = __builtin_fmaf(n1[2], e1[2], __builtin_fmaf(n1[1], e1[1], n1[0] * e1[0]));
+    float out[24];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        out[12 + a] = n0[a];
-        out[15 + a] = n1[a];
+        out[a] = c[0][a];
+        out[3 + a] = e1[a];
+        out[6 + a] = e2[a];
+        out[9 + a] = e3[a];
+        out[12 + a] = n1[a];
+        out[16 + a] = n0[a];
+        out[19 + a] = n2[a];
     }
-    out[18] = __uint_as_float(g);
-    out[19] = 0.f;
+    out[15] = __uint_as_float(g);
+    out[22] = c1;
+    out[23] = 0.f;
     float4 *dst = reinterpret_cast<float4 *>(&leaves[i]);
 #pragma unroll
-    for (int k = 0; k < 5; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
+    for (int k = 0; k < 6; ++k) dst[k] = make_float4(out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]);
 
     // the conservative stand-in (see DstLeafPre): mean plane, averaged half edges, their dual vectors
     float cen[3], nrm[3], h1[3], h2[3];
@@ -862,8 +868,8 @@ __global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const 
 // agent-scope protocol through memory, whose fences write back and invalidate the L2 of the XCD.
 constexpr int kFitBlock = 1024;
 __global__ __launch_bounds__(kFitBlock) void k_fit(DstNode *nodes, const uint32_t *__restrict__ node_parent,
-                      const uint32_t *__restrict__ leaf_parent, uint32_t *flags, const DstLeaf *__restrict__ leaves,
-                      uint32_t n) {
+                      const uint32_t *__restrict__ leaf_parent, uint32_t *flags, const float *__restrict__ vertices,
+                      const int4 *__restrict__ quad_ids, const uint32_t *__restrict__ sorted_ids, uint32_t n) {
     __shared__ float s_box[kFitBlock][12];      // per local node: box of child 0, box of child 1
     __shared__ uint32_t s_arrived[kFitBlock];
     s_arrived[threadIdx.x] = 0u;
@@ -871,13 +877,10 @@ __global__ __launch_bounds__(kFitBlock) void k_fit(DstNode *nodes, const uint32_
     const uint32_t blk_lo = blockIdx.x * blockDim.x, blk_hi = min(blk_lo + blockDim.x, n) - 1u;
     uint32_t i = blk_lo + threadIdx.x;
     if (i >= n) return;
-    const DstLeaf &L = leaves[i];
     float box[6];
     float c[4][3];
-#pragma unroll
-    for (int a = 0; a < 3; ++a) {
-        c[0][a] = L.A[a]; c[1][a] = L.B[a]; c[2][a] = L.C[a]; c[3][a] = L.D[a];
-    }
+    const uint32_t g = sorted_ids[i];
+    load_corners(vertices, quad_ids[g], g, c);   // (the leaf records hold edge vectors, not the corners)
     const float pad = kBoxPad * quad_magnitude(c);   // as in wave_range_boxes: the two fits give the same bits
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -1323,8 +1326,9 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
             hipLaunchKernelGGL(k_fit_ranges, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, rb, n_blocks, n - 1);
     } else {
         hipLaunchKernelGGL(k_fill_u32, grid_for(n), dim3(kBlock), 0, stream, fit_flags, 0u, n);
+        if (vertices == nullptr) return dst_fail(ctx, DST_E_INVALID, "the fit by arrival counters reads the corners from a vertex buffer");
         hipLaunchKernelGGL(k_fit, dim3((n + kFitBlock - 1) / kFitBlock), dim3(kFitBlock), 0, stream, ctx->nodes, ctx->node_parent, ctx->leaf_parent,
-                           fit_flags, ctx->leaves, n);
+                           fit_flags, vertices, quad_ids, ctx->vals[0], n);
     }
     if (n > DST_GROUP)
         hipLaunchKernelGGL(k_widen, grid_for(n - 1), dim3(kBlock), 0, stream, ctx->nodes, ctx->wide, n - 1, ctx->ploc_state + 5);

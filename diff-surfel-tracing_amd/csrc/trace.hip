@@ -172,27 +172,32 @@ __device__ __forceinline__ F3 cross_f(F3 x, F3 y) {
 __device__ __forceinline__ float dot_f(F3 a, F3 b) {
     return __builtin_fmaf(a.z, b.z, __builtin_fmaf(a.y, b.y, a.x * b.x));
 }
-__device__ __forceinline__ float triple(F3 d, F3 x, F3 y) { return dot_f(d, cross_f(x, y)); }
 __device__ __forceinline__ bool same_sign(float a, float b, float c) {
     return (a >= 0.f && b >= 0.f && c >= 0.f) || (a <= 0.f && b <= 0.f && c <= 0.f);
 }
-// Quad = triangles ABC and BCD with plane normals n0, n1.  Signed-volume edge tests in origin-relative
-// coordinates, then t = n.(v1-o) / n.d on the plane of the triangle that was hit.
-__device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 B, F3 C, F3 Dv, F3 n0, F3 n1, float &t, uint32_t &tri) {
-    F3 a = A - o, b = B - o, c = C - o, e = Dv - o;
-    float u0 = triple(d, b, c);
-    float u1 = triple(d, c, a);
-    float u2 = triple(d, a, b);
-    bool in0 = same_sign(u0, u1, u2);
-    float w0 = triple(d, c, e);
-    float w1 = triple(d, e, b);
-    bool in1 = same_sign(w0, w1, u0);
+// Quad = triangles ABC and BCD, given as the leaf record holds it: corner A, edge vectors AB, AC, AD, normals
+// n0 = AB x AC, n1 = (C-B) x (D-B), n2 = AC x AD, c1 = n1.AB.  The signed volumes d.((P-o) x (Q-o)) of the edge tests
+// are formed from one cross product with the ray, m = d x (A-o), and the edge vectors:
+//     d.((A+P'-o) x (A+Q'-o)) = (Q'-P').m + d.(P' x Q'),
+// so that nothing is multiplied that is as long as the way from the origin to the quad except in m itself (with the
+// corners relative to the origin in every product, a ray passing half a millimetre-sized quad outside it counted as
+// a hit from a few metres away).  Then t = n.(v1-o) / n.d on the plane of the triangle that was hit.
+__device__ __forceinline__ bool ray_quad(F3 o, F3 d, F3 A, F3 AB, F3 AC, F3 AD, F3 n0, F3 n1, F3 n2, float c1, float &t,
+                                         uint32_t &tri) {
+    const F3 a = A - o;
+    const F3 m = cross_f(d, a);
+    const float X = dot_f(AB, m), Y = dot_f(AC, m), Z = dot_f(AD, m);
+    const float q0 = dot_f(n0, d), q1 = dot_f(n1, d), q2 = dot_f(n2, d);
+    const float u2 = X, u1 = -Y, u0 = (Y - X) + q0;          // edges AB, CA, BC
+    const bool in0 = same_sign(u0, u1, u2);
+    const float w0 = (Z - Y) + q2;                            // edge CD
+    const float w1 = (X - Z) + ((q1 - q0) - q2);              // edge DB (AD x AB = n1 - n0 - n2)
+    const bool in1 = same_sign(w0, w1, u0);
     if (!(in0 || in1)) return false;
-    F3 n = in0 ? n0 : n1;
-    F3 k = in0 ? a : b;
     tri = in0 ? 0u : 1u;
-    float p = dot_f(n, k);
-    float q = dot_f(n, d);
+    const float pa = dot_f(in0 ? n0 : n1, a);
+    const float p = in0 ? pa : pa + c1;                       // n1.(B-o) = n1.(A-o) + n1.AB
+    const float q = in0 ? q0 : q1;
     t = p / q;
     return (t > 0.0f) && (t < kInfDepth);
 }
@@ -231,7 +236,7 @@ __device__ __forceinline__ void load_node(const void *node, uint32_t onx, uint32
         : "s"(node), "s"(onx), "s"(ony), "s"(onz), "s"(ofx), "s"(ofy), "s"(ofz)
         : "memory");
 }
-// Two consecutive 64-byte records (the stand-ins of a leaf group's two quads), or one 80-byte quad record, in one
+// Two consecutive 64-byte records (the stand-ins of a leaf group's two quads), or one 96-byte quad record, in one
 // trip: left to itself the compiler splits these fetches and waits for the first part before asking for the rest.
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ void load_record_pair(const void *p, u32x16 &a, u32x16 &b) {
@@ -240,8 +245,9 @@ __device__ __forceinline__ void load_record_pair(const void *p, u32x16 &a, u32x1
                  : "s"(p)
                  : "memory");
 }
-__device__ __forceinline__ void load_quad_record(const void *p, u32x16 &a, u32x4 &b) {
-    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx4 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ void load_quad_record(const void *p, u32x16 &a, u32x8 &b) {
+    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx8 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
                  : "=&s"(a), "=&s"(b)
                  : "s"(p)
                  : "memory");
@@ -424,19 +430,20 @@ __device__ __forceinline__ uint64_t quad_may_hit(const u32x16 &Q, const RayPre &
 }
 
 // The exact test of one quad record for all lanes; hits are admitted into the lanes' buffers.
-__device__ __forceinline__ void quad_exact(const u32x16 &La, const u32x4 &Lb, F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
+__device__ __forceinline__ void quad_exact(const u32x16 &La, const u32x8 &Lb, F3 o, F3 d, bool active, KBuf &buf, uint32_t &cnt
 #ifdef DST_STATS
                                            , WaveStats &ws
 #endif
 ) {
     STAT(ws.t_plan++;)
-#define LW(k) ((k) < 16 ? La[(k) & 15] : Lb[((k) - 16) & 3])
+#define LW(k) ((k) < 16 ? La[(k) & 15] : Lb[((k) - 16) & 7])
 #define LF3(k) f3(__uint_as_float(LW(k)), __uint_as_float(LW((k) + 1)), __uint_as_float(LW((k) + 2)))
     float t = 0.f;
     uint32_t tri = 0u;
-    const bool hit = active && ray_quad(o, d, LF3(0), LF3(3), LF3(6), LF3(9), LF3(12), LF3(15), t, tri);
+    const bool hit = active && ray_quad(o, d, LF3(0), LF3(3), LF3(6), LF3(9), LF3(16), LF3(12), LF3(19),
+                                        __uint_as_float(LW(22)), t, tri);
 #undef LF3
-    const uint64_t x = kb_pack(t, 2u * LW(18) + tri);
+    const uint64_t x = kb_pack(t, 2u * LW(15) + tri);
 #undef LW
     const bool adm = hit && (x < buf.e[kChunk - 1]);
     if (wave_ballot(adm) != 0ull) {
@@ -478,7 +485,7 @@ __device__ __forceinline__ bool test_group(const DstAccelView &acc, uint32_t fir
             const uint32_t k = (todo & 1u) ? 0u : 1u;
             todo &= ~(1u << k);
             u32x16 La;
-            u32x4 Lb;
+            u32x8 Lb;
             load_quad_record(&acc.leaves[first + q0 + k], La, Lb);
             quad_exact(La, Lb, o, d, active, buf, cnt WSP);
         }
@@ -702,7 +709,7 @@ typedef const __attribute__((address_space(1))) uint32_t *global_u32;
 constexpr int kLaneShelf = 32;
 struct LaneWalkAccel { const DstLeaf *leaves; const DstWideNode *wide; uint32_t n_leaves, root; };   // by value: registers
 static_assert(DST_GROUP <= 2, "the per-lane walk fetches a leaf group as at most two quad records");
-static_assert(sizeof(DstWideNode) == 128 && sizeof(DstLeaf) == 80, "the per-lane walk reads both as 16-byte words");
+static_assert(sizeof(DstWideNode) == 128 && sizeof(DstLeaf) == 96, "the per-lane walk reads both as 16-byte words");
 // A value that is the same in every lane, moved to a scalar register (arguments of a real call arrive in vector ones).
 template <class T>
 __device__ __forceinline__ T *uniform_ptr(T *p) {
@@ -730,11 +737,11 @@ __device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc_in, 
     uint32_t ref = active ? acc.root : kWalkDone;
     uint32_t budget = 2u * acc.n_leaves + 8u;   // a well-formed hierarchy needs fewer steps; bounds the loop regardless
     // A step of a lane is one dependent trip to memory: the lane's node (128 bytes) or its leaf group (two quad
-    // records of 80 bytes, consecutive) is requested whole - eight to ten 16-byte loads from one base address, whatever
+    // records of 96 bytes, consecutive, the first 64 of each) is requested whole - eight to ten 16-byte loads from one base address, whatever
     // the lane is at - before anything is tested, so that lanes at nodes and lanes at leaf groups wait together,
-    // once.  (Left to the compiler, a quad came in three trips - corners A to C, then D and the normals behind the
-    // first edge test, then the surfel id behind the hit - and the lanes at leaf groups took theirs after the lanes
-    // at nodes had finished theirs.)
+    // once.  (Left to the compiler, a quad came in three trips - the first words, then the rest behind the first edge
+    // test, then the surfel id behind the hit - and the lanes at leaf groups took theirs after the lanes at nodes had
+    // finished theirs.)
     typedef const __attribute__((address_space(1))) v4f *global_v4f;
 #pragma unroll 1
     while (wave_ballot(ref != kWalkDone) != 0ull) {
@@ -748,8 +755,8 @@ __device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc_in, 
             const bool two = is_leaf && count > 1u && first + 1u < acc.n_leaves;
             const global_v4f src = is_leaf ? (global_v4f)reinterpret_cast<const v4f *>(&acc.leaves[first])
                                            : (global_v4f)reinterpret_cast<const v4f *>(&acc.wide[ref]);
-            // a node is 8 x 16 bytes; one quad is 5 (a leaf group of one quad asks for 8 as well: the array has spare
-            // records behind its last quad), two quads are 10
+            // a node is 8 x 16 bytes; of a quad's record the first 4 words of 16 bytes are read (a leaf group of one quad
+            // asks for 8 as well: the array has spare records behind its last quad), the second quad's are words 6 to 9
             v4f r0 = src[0], r1 = src[1], r2 = src[2], r3 = src[3], r4 = src[4], r5 = src[5], r6 = src[6], r7 = src[7];
             v4f r8 = {0.f, 0.f, 0.f, 0.f}, r9 = {0.f, 0.f, 0.f, 0.f};
             if (two) {
@@ -760,28 +767,24 @@ __device__ __attribute__((noinline)) void lane_walk(const LaneWalkAccel acc_in, 
             asm volatile("" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4));
             asm volatile("" : "+v"(r5), "+v"(r6), "+v"(r7), "+v"(r8), "+v"(r9));
             if (is_leaf) {
-                {
-                    float t = 0.f;
-                    uint32_t tri = 0u;
-                    const bool hit = ray_quad(o, d, f3(r0.x, r0.y, r0.z), f3(r0.w, r1.x, r1.y), f3(r1.z, r1.w, r2.x),
-                                              f3(r2.y, r2.z, r2.w), f3(r3.x, r3.y, r3.z), f3(r3.w, r4.x, r4.y), t, tri);
-                    const uint64_t x = kb_pack(t, 2u * __float_as_uint(r4.z) + tri);
-                    if (hit && (x < buf.e[kChunk - 1])) {
-                        cnt += 1u;
-                        kbuf_insert(buf, x, true);
-                    }
-                }
-                if (two) {
-                    float t = 0.f;
-                    uint32_t tri = 0u;
-                    const bool hit = ray_quad(o, d, f3(r5.x, r5.y, r5.z), f3(r5.w, r6.x, r6.y), f3(r6.z, r6.w, r7.x),
-                                              f3(r7.y, r7.z, r7.w), f3(r8.x, r8.y, r8.z), f3(r8.w, r9.x, r9.y), t, tri);
-                    const uint64_t x = kb_pack(t, 2u * __float_as_uint(r9.z) + tri);
-                    if (hit && (x < buf.e[kChunk - 1])) {
-                        cnt += 1u;
-                        kbuf_insert(buf, x, true);
-                    }
-                }
+                // the first 64 bytes of a record: A, AB, AC, AD, n1 (three floats each), surfel id; n0, n2 and c1 are
+                // formed as the builder forms them for the record's other 32 bytes
+#define DST_LANE_QUAD(w0, w1, w2, w3)                                                                                  \
+    {                                                                                                                  \
+        float t = 0.f;                                                                                                 \
+        uint32_t tri = 0u;                                                                                             \
+        const F3 AB = f3(w0.w, w1.x, w1.y), AC = f3(w1.z, w1.w, w2.x), AD = f3(w2.y, w2.z, w2.w), n1 = f3(w3.x, w3.y, w3.z); \
+        const bool hit = ray_quad(o, d, f3(w0.x, w0.y, w0.z), AB, AC, AD, cross_f(AB, AC), n1, cross_f(AC, AD),        \
+                                  dot_f(n1, AB), t, tri);                                                              \
+        const uint64_t x = kb_pack(t, 2u * __float_as_uint(w3.w) + tri);                                               \
+        if (hit && (x < buf.e[kChunk - 1])) {                                                                          \
+            cnt += 1u;                                                                                                 \
+            kbuf_insert(buf, x, true);                                                                                 \
+        }                                                                                                              \
+    }
+                DST_LANE_QUAD(r0, r1, r2, r3)
+                if (two) DST_LANE_QUAD(r6, r7, r8, r9)
+#undef DST_LANE_QUAD
                 // (groups of more than two quads do not occur: DST_GROUP = 2; a longer one would lose its tail)
             } else {
                 // lox r0, loy r1, loz r2, hix r3, hiy r4, hiz r5, child references r6, child count r7.x

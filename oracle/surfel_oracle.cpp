@@ -24,8 +24,9 @@
  * because no source for them exists to follow -- parity of these against OptiX
  * itself is UNPINNED:
  *   - the set of hits of a ray: every surfel quad (two triangles sharing the
- *     edge B-C) is tested with signed-volume edge functions in ray-origin
- *     relative coordinates (cross and dot products with fused multiply-adds,
+ *     edge B-C) is tested with signed-volume edge functions, formed from the
+ *     cross product of the ray with corner A relative to the origin and the
+ *     quad's edge vectors (cross and dot products with fused multiply-adds,
  *     written out in ray_quad()); at most one hit per quad; triangle 0 wins
  *     ties on the shared edge;
  *   - the hit parameter: t = n.(v1-o) / n.d with n = (v2-v1)x(v3-v1) of the hit
@@ -254,30 +255,38 @@ inline V3 cross_f(V3 x, V3 y) {
     return V3{std::fmaf(x.y, y.z, -(x.z * y.y)), std::fmaf(x.z, y.x, -(x.x * y.z)), std::fmaf(x.x, y.y, -(x.y * y.x))};
 }
 inline float dot_f(V3 a, V3 b) { return std::fmaf(a.z, b.z, std::fmaf(a.y, b.y, a.x * b.x)); }
-inline float triple(V3 d, V3 x, V3 y) { return dot_f(d, cross_f(x, y)); }
 inline bool same_sign(float a, float b, float c) {
     return (a >= 0.f && b >= 0.f && c >= 0.f) || (a <= 0.f && b <= 0.f && c <= 0.f);
 }
+// Quad = triangles ABC and BCD.  With a = A - o, m = d x a and the edge vectors AB, AC, AD from corner A, the signed
+// volume of an edge test is  d.((A+P'-o) x (A+Q'-o)) = (Q'-P').m + d.(P' x Q'):  the only product of two vectors as
+// long as the way from the origin to the quad is m itself, so the test decides to within about eps |a| of an edge.
+// (Formed from the four corners relative to the origin, the volumes carry an error of eps |a|^2 / |edge|: half a quad's
+// width for millimetre quads seen from a few metres.)  Everything that depends on the quad alone - the edge vectors,
+// n0 = AB x AC, n1 = (C-B) x (D-B), n2 = AC x AD, c1 = n1.AB - is what the library keeps per quad.
 inline bool ray_quad(V3 o, V3 d, V3 A, V3 B, V3 C, V3 Dv, float &t, int &tri) {
-    V3 a = A - o, b = B - o, c = C - o, e = Dv - o;
-    float u0 = triple(d, b, c);
-    float u1 = triple(d, c, a);
-    float u2 = triple(d, a, b);
-    V3 n, k;
+    const V3 AB = B - A, AC = C - A, AD = Dv - A;
+    const V3 n0 = cross_f(AB, AC), n1 = cross_f(C - B, Dv - B), n2 = cross_f(AC, AD);
+    const float c1 = dot_f(n1, AB);
+    const V3 a = A - o;
+    const V3 m = cross_f(d, a);
+    const float X = dot_f(AB, m), Y = dot_f(AC, m), Z = dot_f(AD, m);
+    const float q0 = dot_f(n0, d), q1 = dot_f(n1, d), q2 = dot_f(n2, d);
+    const float u2 = X, u1 = -Y, u0 = (Y - X) + q0;   // edges AB, CA, BC
+    float p, q;
     if (same_sign(u0, u1, u2)) {
-        n = cross_f(B - A, C - A);
-        k = a;
+        p = dot_f(n0, a);
+        q = q0;
         tri = 0;
     } else {
-        float w0 = triple(d, c, e);
-        float w1 = triple(d, e, b);
+        const float w0 = (Z - Y) + q2;                  // edge CD
+        const float w1 = (X - Z) + ((q1 - q0) - q2);    // edge DB: AD x AB = n1 - n0 - n2
         if (!same_sign(w0, w1, u0)) return false;
-        n = cross_f(C - B, Dv - B);
-        k = b;
+        const float pa = dot_f(n1, a);
+        p = pa + c1;                                    // n1.(B-o)
+        q = q1;
         tri = 1;
     }
-    float p = dot_f(n, k);
-    float q = dot_f(n, d);
     t = p / q;
     return (t > 0.0f) && (t < kInfDepth);
 }

@@ -90,9 +90,17 @@ uint32_t check_structure(const dst_ctx &c, const Scene &s, const char *what) {
         CHECK(L.g < n, "%s: leaf %u holds surfel %u", what, i, L.g);
         if (L.g >= n) continue;
         seen[L.g]++;
-        CHECK(std::memcmp(L.A, &s.v[12 * (size_t)L.g], 48) == 0, "%s: corners of leaf %u", what, i);
+        {   // corner A and the edge vectors to B, C, D, as the fp32 differences of the corners
+            const float *v = &s.v[12 * (size_t)L.g];
+            float want[12];
+            for (int a = 0; a < 3; ++a) {
+                want[a] = v[a];
+                for (int k = 1; k < 4; ++k) want[3 * k + a] = v[3 * k + a] - v[a];
+            }
+            CHECK(std::memcmp(L.A, want, 48) == 0, "%s: corner and edges of leaf %u", what, i);
+        }
         float cc[4][3];
-        std::memcpy(cc, L.A, 48);
+        std::memcpy(cc, &s.v[12 * (size_t)L.g], 48);
         float mag = 0.f;
         for (int k = 0; k < 4; ++k)
             for (int a = 0; a < 3; ++a)

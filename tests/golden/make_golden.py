@@ -3,7 +3,8 @@ differ in the last bit between CPUs) and the expected outputs from the CPU oracl
 enumeration, reference any-hit rule).  The reference ships no golden vectors and cannot be
 run here (it needs nvcc + OptiX), so this fixture pins the oracle against later drift, not against the reference.
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            (keeps the stored inputs of an existing fixture, renews the outputs)
+    python tests/golden/make_golden.py --new-inputs
 """
 import os
 import sys
@@ -41,7 +42,8 @@ def inputs():
 def main():
     from helpers import oracle_scene
     from oracle import surfel_oracle as O
-    sc, o, d, ug = inputs()
+    keep = os.path.exists(os.path.join(HERE, "cube_p400.npz")) and "--new-inputs" not in sys.argv
+    sc, o, d, ug = load_inputs() if keep else inputs()
     s = oracle_scene(O, sc, o, d, bg=SPEC["bg"])
     fwd = O.forward(s, O.HITS_BRUTE_LITERAL)
     bwd = O.backward(s, fwd, {k: v.numpy() for k, v in ug.items()}, O.HITS_BRUTE_LEXI)

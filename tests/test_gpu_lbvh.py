@@ -13,15 +13,15 @@ LEAF = 0x80000000
 
 NODE = np.dtype([("lo0", "<f4", 3), ("hi0", "<f4", 3), ("lo1", "<f4", 3), ("hi1", "<f4", 3), ("c0", "<u4"),
                  ("c1", "<u4"), ("first", "<u4"), ("last", "<u4")])
-LEAFT = np.dtype([("A", "<f4", 3), ("B", "<f4", 3), ("C", "<f4", 3), ("D", "<f4", 3), ("n0", "<f4", 3),
-                  ("n1", "<f4", 3), ("g", "<u4"), ("pad", "<u4")])
+LEAFT = np.dtype([("A", "<f4", 3), ("AB", "<f4", 3), ("AC", "<f4", 3), ("AD", "<f4", 3), ("n1", "<f4", 3),
+                  ("g", "<u4"), ("n0", "<f4", 3), ("n2", "<f4", 3), ("c1", "<f4"), ("pad", "<u4")])
 
 
 def download(tracer):
     import diff_surfel_tracing._C as binding
     ctx = tracer.optix_context
     info = ctx.accel_info()
-    assert info.node_bytes == NODE.itemsize == 64 and info.leaf_bytes == LEAFT.itemsize == 80
+    assert info.node_bytes == NODE.itemsize == 64 and info.leaf_bytes == LEAFT.itemsize == 96
     n = info.n_surfels
     nodes = np.zeros(max(n - 1, 1), NODE)
     leaves = np.zeros(n, LEAFT)
@@ -63,21 +63,30 @@ def check_tree(info, nodes, leaves, npar, lpar, keys, vertices):
         assert bool(c0 & LEAF) == (split == f) and bool(c1 & LEAF) == (split + 1 == l)
     assert sorted(leaves["g"].tolist()) == list(range(n))              # every surfel exactly once
     V = vertices.reshape(n, 4, 3)
-    for name, k in (("A", 0), ("B", 1), ("C", 2), ("D", 3)):
-        np.testing.assert_array_equal(leaves[name], V[leaves["g"], k])
-    A, B, C, D = (leaves[c].astype(np.float64) for c in "ABCD")
-    np.testing.assert_allclose(leaves["n0"], np.cross(B - A, C - A), rtol=1e-4, atol=1e-7)   # plane normals
-    np.testing.assert_allclose(leaves["n1"], np.cross(C - B, D - B), rtol=1e-4, atol=1e-7)
+    corners = {name: V[leaves["g"], k] for name, k in (("A", 0), ("B", 1), ("C", 2), ("D", 3))}
+    np.testing.assert_array_equal(leaves["A"], corners["A"])           # corner A and the edge vectors from it, as
+    with np.errstate(invalid="ignore"):                                # the fp32 differences of the corners
+        for name, k in (("AB", "B"), ("AC", "C"), ("AD", "D")):
+            np.testing.assert_array_equal(leaves[name], corners[k] - corners["A"])
+    A, B, C, D = (corners[c].astype(np.float64) for c in "ABCD")
+    with np.errstate(invalid="ignore"):
+        np.testing.assert_allclose(leaves["n0"], np.cross(B - A, C - A), rtol=1e-4, atol=1e-7)   # plane normals
+        np.testing.assert_allclose(leaves["n1"], np.cross(C - B, D - B), rtol=1e-4, atol=1e-7)
+        np.testing.assert_allclose(leaves["n2"], np.cross(C - A, D - A), rtol=1e-4, atol=1e-7)
+        n1 = np.cross(C - B, D - B)                                    # (c1 = n1.AB is all cancellation on a flat quad)
+        scale = np.linalg.norm(n1, axis=1) * np.linalg.norm(B - A, axis=1)
+        ok = np.isfinite(scale)
+        assert (np.abs(leaves["c1"] - (n1 * (B - A)).sum(1))[ok] <= 1e-5 * scale[ok] + 1e-30).all()
     # a leaf's box: its corners, widened by 4e-6 of the quad's largest coordinate (the quad's share of the slack the
     # box tests need; computed in fp32 like the kernel does)
     with np.errstate(invalid="ignore"):
         mag = np.zeros(n, np.float32)
         for c in "ABCD":
-            a = np.abs(leaves[c])
+            a = np.abs(corners[c])
             mag = np.maximum(mag, np.where(np.isfinite(a), a, np.float32(0)).max(1))
     pad = (np.float32(4e-6) * mag)[:, None]
-    llo = np.minimum.reduce([leaves[c] for c in "ABCD"]) - pad
-    lhi = np.maximum.reduce([leaves[c] for c in "ABCD"]) + pad
+    llo = np.minimum.reduce([corners[c] for c in "ABCD"]) - pad
+    lhi = np.maximum.reduce([corners[c] for c in "ABCD"]) + pad
     assert llo.dtype == np.float32 and lhi.dtype == np.float32
     # walk from the root: every node and leaf reached once, parents consistent, boxes = exact union of content
     seen_nodes, seen_leaves = np.zeros(n - 1, bool), np.zeros(n, bool)
