@@ -29,9 +29,7 @@ def handed(tracer):
 def ball_scene(P=170000, n_ball=150000, radius=0.06, centre=(1.0, 0.5, 0.0), shrink=0.018, seed=0):
     """The 10 m room with most of its surfels moved into a ball of 12 cm and shrunk to 2 mm quads: seen from half a
     metre away at 64x64 pixels, an 8x8 tile's frustum holds some ten thousand quads, each wanted by one ray at best.
-    (Sizes chosen so that the quad test still decides far from its rounding: with quads of a tenth of that size seen
-    from several metres, a ray passing half a quad outside one can count as a hit of it - for a walk that tests
-    every quad, and for no walk that culls by boxes.)"""
+    (Smaller quads seen from farther away: test_submillimetre_quads_seen_from_metres_away.)"""
     sc = S.scene_room(P=P, seed=seed)
     gen = torch.Generator().manual_seed(seed + 1)
     idx = torch.randperm(P, generator=gen)[:n_ball]
@@ -93,6 +91,38 @@ def test_dense_ball_of_subpixel_quads_is_handed_over_by_default(oracle):
         times[mode] = forward_ms(tracer, sc, o, d)
     print("dense ball, forward: %.2f ms handed over, %.2f ms without" % (times["auto"], times["off"]), flush=True)
     assert times["auto"] < 0.75 * times["off"]
+
+
+def test_submillimetre_quads_seen_from_metres_away(oracle):
+    """Quads of about 1 mm, 3.4 m from the camera: the quad test has to decide them to a small fraction of their size,
+    or a walk that tests every quad and walks that cull by boxes see different hits.  Brute force, the oracle's BVH
+    and both GPU walks agree bit for bit."""
+    P, n_ball = 200000, 180000
+    sc = S.scene_room(P=P, seed=0)
+    gen = torch.Generator().manual_seed(1)
+    idx = torch.randperm(P, generator=gen)[:n_ball]
+    centre = torch.tensor([1.0, 0.5, 0.0])
+    sc["means3D"][idx] = sc["means3D"][idx] * 0.01 + centre
+    sc["scales"][idx] *= 0.01
+    sc["vertices"], sc["faces"] = S.get_triangles(sc["means3D"], sc["scales"], sc["rotations"])
+    o, d = S.rays_room(540, 960)
+    r, c = divmod(int((d * torch.nn.functional.normalize(centre - o[0, 0], dim=0)).sum(-1).argmax()), 960)
+    r0, c0 = r - r % 8 - 16, c - c % 8 - 16
+    o, d = o[r0:r0 + 32, c0:c0 + 32].contiguous(), d[r0:r0 + 32, c0:c0 + 32].contiguous()
+    assert float((centre - o[0, 0]).norm()) > 3.0 and float(6 * sc["scales"][idx].median()) < 1.5e-3
+    ref = oracle.forward(oracle_scene(oracle, sc, o, d), oracle.HITS_BVH_LEXI)
+    mid = slice(8, 24)
+    brute = oracle.forward(oracle_scene(oracle, sc, o[mid, mid].contiguous(), d[mid, mid].contiguous()),
+                           oracle.HITS_BRUTE_LEXI)
+    for k in ("rgb", "dpt", "acc", "norm"):
+        assert np.array_equal(brute[k].view(np.uint32), ref[k][mid, mid].view(np.uint32)), k
+    assert ref["n_con"][mid, mid].mean() > 8
+    for mode, steps in (("off", 0), ("always", 256)):
+        tracer = own_tracer(mode, steps)
+        before = handed(tracer)
+        out, _ = gpu_trace(tracer, sc, o, d, training=False)
+        assert_forward_exact(out, ref)
+        assert (handed(tracer) > before) == (mode == "always")
 
 
 def test_ordinary_scenes_leave_the_hand_over_off(tracer):

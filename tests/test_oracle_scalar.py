@@ -167,6 +167,49 @@ def test_ray_quad_matches_float64_triangle_tests(oracle):
     assert n_hit > 500 and n_checked > 3000
 
 
+def test_ray_quad_decides_millimetre_quads_seen_from_metres_like_float64(oracle):
+    """The edge tests are formed from one cross product with the ray and the quad's edge vectors, so their error is
+    that of the way to the quad (eps * distance), not of its square over the edge: a 1 mm quad 3 to 6 m away is decided
+    like float64 decides it as soon as the ray is 1 % of the quad away from an edge.  (With the four corners relative to
+    the origin in every product, rays half a quad outside counted as hits at these sizes.)"""
+    rng = np.random.default_rng(5)
+    n_checked = n_hit = n_near = 0
+    for _ in range(6000):
+        c = rng.uniform(-2, 2, 3)
+        e1 = rng.normal(size=3)
+        e1 *= 1e-3 / np.linalg.norm(e1)
+        e2 = np.cross(e1, rng.normal(size=3))
+        e2 *= 1e-3 / np.linalg.norm(e2)
+        A, B, C = c, c + e1, c + e2
+        D = B + (C - A) + 2e-5 * rng.normal(size=3)          # a parallelogram, a little bent
+        A, B, C, D = [x.astype(np.float32).astype(np.float64) for x in (A, B, C, D)]
+        o = c + rng.normal(size=3) * 2.5
+        if np.linalg.norm(o - c) < 3.0:
+            o = c + (o - c) * 3.0 / np.linalg.norm(o - c)
+        target = A + rng.uniform(-0.5, 1.5) * (B - A) + rng.uniform(-0.5, 1.5) * (C - A)
+        d = (target - o) / np.linalg.norm(target - o)
+        o32, d32 = o.astype(np.float32), d.astype(np.float32)
+        hit, t, tri = oracle.ray_quad(o32, d32, *[x.astype(np.float32) for x in (A, B, C, D)])
+        o64, d64 = o32.astype(np.float64), d32.astype(np.float64)
+        inside, margin = [], []
+        for r in (_mt64(o64, d64, A, B, C), _mt64(o64, d64, B, C, D)):
+            tt, u, v = r
+            m = min(u, v, 1 - u - v)
+            inside.append(m >= 0 and tt > 0)
+            margin.append(abs(m))
+        if abs(np.cross(B - A, C - A) @ d64) < 0.2 * 1e-6:   # grazing: the plane hit itself is ill-conditioned
+            continue
+        if min(margin) < 1e-2:
+            continue
+        n_checked += 1
+        n_near += min(margin) < 0.3
+        assert hit == (inside[0] or inside[1]), (margin, inside, hit)
+        if hit:
+            n_hit += 1
+            assert tri == (0 if inside[0] else 1)
+    assert n_checked > 4000 and n_hit > 1000 and n_near > 2000
+
+
 def test_ray_quad_known_answers(oracle):
     A, B, C, D = [np.array(p, np.float32) for p in ([-3, 3, 0], [-3, -3, 0], [3, 3, 0], [3, -3, 0])]
     down = np.array([0, 0, -1], np.float32)
