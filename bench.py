@@ -291,7 +291,10 @@ def run_workload(key, steps, warmup, main, args):
 
     aux_max = 2 if aux_out <= 2 else (4 if aux_out <= 4 else 8)
     mixed = "true" if (depth > 0 or H < 8) else "false"   # kernels with the per-lane walk built in
-    fwd_roof = roofline_of(key, "forward", "k_trace_fwd<%d,true,%s,false>" % (aux_max, mixed), A_fwd, fwd_ms,
+    # (image grids at depth 0 run the kernels without the tile hand-over unless the scene has many small quads)
+    fwd_name = ("k_trace_fwd_plain<%d,true>" % aux_max if mixed == "false" and not trace_info.handover_active
+                else "k_trace_fwd<%d,true,%s,false>" % (aux_max, mixed))
+    fwd_roof = roofline_of(key, "forward", fwd_name, A_fwd, fwd_ms,
                            "per ray / evaluated entry / composited hit, reference-shaped")
     bwd_roof = roofline_of(key, "backward", "k_trace_bwd<%d,true,false,false>" % aux_max, A_replay, bwd_ms,
                            "what the replaying kernel moves by design: record, per-hit geometry, gradient rows")
