@@ -151,7 +151,6 @@ struct dst_ctx {
     uint32_t handover_steps = kDstHandoverSteps;   // limit of a tile's first walk
     int handover_mode = DST_HANDOVER_AUTO;         // auto: only for scenes with many small quads
     uint32_t small_quads = 0;          // as counted by the last build
-    uint32_t handover_parity = 0;      // which of the list's two counters the next trace counts in
     DstBounds *bounds = nullptr;       // device (allocated by dst_create together with the hand-over list)
     DstBounds *bounds_host = nullptr;  // pinned host copy
     void *core_box = nullptr;          // device: the box the two-level Morton keys are laid over (lbvh.hip)

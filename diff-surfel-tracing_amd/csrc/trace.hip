@@ -1902,14 +1902,15 @@ __global__ __launch_bounds__(1024) void k_block_order(const uint32_t *__restrict
 // Tile hand-over (forward).  A packet walk visits what any of its 64 rays needs, one dependent fetch after the other.
 // Over geometry much finer than the ray spacing (a dense cloud of surfels far smaller than a pixel) that is the whole
 // content of the tile's frustum, wanted by one ray at best, and a single wave walks for milliseconds while the chip
-// idles.  So the first walk of a tile may take `hand_arg` steps (bits 0..30) and no more: a wave that runs into that
-// limit has written nothing yet, puts its tile on the context's list and leaves, and a second, small launch right
-// behind (kernels with the per-lane walk, hand_arg steps = 0: the takers) traces the listed tiles with every ray
-// walking on its own - the same buffer content, so the same results bit for bit.  List: word 0 / 1 = tiles listed by
-// the trace of even / odd parity (hand_arg bit 31; a trace's takers clear the word the next trace will count in),
-// word 2 = tiles handed over since the context was made, entries ((by * btiles_x + bx) * 4 + wave) from word 4.  A
-// wave that finds the list full starts again without a limit.
-constexpr uint32_t kHandHeader = kDstHandoverHeader, kHandCap = kDstHandoverCap, kHandStepsMask = 0x7FFFFFFFu;
+// idles.  So the first walk of a tile may take `hand_arg` steps and no more: a wave that runs into that limit has
+// written nothing yet, puts its tile on the context's list and leaves, and a second, small launch right behind
+// (kernels with the per-lane walk, hand_arg = 0: the takers) traces the listed tiles with every ray walking on its
+// own - the same buffer content, so the same results bit for bit.  List: word 0 = tiles listed by this trace, word 1 =
+// takers that have read their entry (the last one empties the list for the next trace: nothing on the host changes
+// from call to call, so a captured launch pair can be replayed), word 2 = tiles handed over since the context was
+// made, entries ((by * btiles_x + bx) * 4 + wave) from word 4.  A wave that finds the list full starts again without
+// a limit.
+constexpr uint32_t kHandHeader = kDstHandoverHeader, kHandCap = kDstHandoverCap;
 template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET, bool HAND>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
                                            uint32_t tiles_x, uint32_t tiles_y, uint32_t btiles_x,
@@ -1969,20 +1970,27 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
     if (BWD && block_order != nullptr) bid = block_order[bid];   // replay: the longest blocks first (k_block_order)
     uint32_t bx, by;
     static_assert(!HAND || (!BWD && kFwdWavesPerBlock == 1), "tiles are handed over by forward kernels of one wave per workgroup");
-    const bool taker = HAND && MIXED && handover != nullptr && (hand_arg & kHandStepsMask) == 0u;
+    const bool taker = HAND && MIXED && handover != nullptr && hand_arg == 0u;
     block_of_position(bid, btiles_x, (tiles_y + 1u) / 2u, strip_width, th_log2 != 0, bx, by);
     if constexpr (HAND) {
         if (taker) {   // the tile comes from the list, not from the workgroup's number
-            const uint32_t par = hand_arg >> 31, n = min(handover[par], gridDim.x);
-            if (blockIdx.x == 0u && threadIdx.x == 0u) {
-                handover[par ^ 1u] = 0u;
-                handover[2] += n;
-            }
-            if (blockIdx.x >= n) return;
-            const uint32_t id = handover[kHandHeader + blockIdx.x];
+            const uint32_t n = min(handover[0], gridDim.x);
+            const uint32_t id = handover[kHandHeader + min(blockIdx.x, kHandCap - 1u)];
             wv = id & 3u;
             bx = (id >> 2) % btiles_x;
             by = (id >> 2) / btiles_x;
+            // Every taker has read the count and its entry before it is counted itself (the fence keeps the reads in front
+            // of the ticket), and no wave writes the list while takers run: the last one counted empties it.
+            __threadfence();
+            if (threadIdx.x == 0u) {
+                const uint32_t ticket = atomicAdd(&handover[1], 1u);
+                if (ticket == gridDim.x - 1u) {
+                    handover[2] += n;
+                    handover[1] = 0u;
+                    handover[0] = 0u;
+                }
+            }
+            if (blockIdx.x >= n) return;
         }
     }
     const bool flat = th_log2 == 0;   // a ray list: tiles of 1x64 rays, a block = four consecutive tiles
@@ -2029,14 +2037,14 @@ __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelVie
         F3 ot = ray_o, dt = ray_d;
         float s_prod = 1.0f;
         bool on = inside;
-        uint32_t first_walk = (HAND && handover != nullptr) ? (hand_arg & kHandStepsMask) : 0u;
+        uint32_t first_walk = (HAND && handover != nullptr) ? hand_arg : 0u;
         for (int i = 0; i <= mtd; ++i) {
             const float min_depth = (i == 0) ? (p.start_from_first ? kNear : 0.0f) : kStartOffset;
             F3 dist_acc = f3(0, 0, 0);
             const bool gave_up = walk_bounce<false, AUXM, REC, MIXED, DET, HAND>(p, acc, max_abs, on, ot, dt, min_depth, run, in, g_ro, g_rd, n_proc, n_con, WET ? wet_keys : nullptr, WET ? wet_vals : nullptr, nullptr, rv, i, dist_acc, taker ? kWalkPerLane : (i == 0 ? first_walk : 0u) WS_ARG);
             if constexpr (HAND) if (gave_up) {   // (bounce 0, before anything was written; no else below)
                 uint32_t slot = 0u;
-                if (lane == 0u) slot = atomicAdd(&handover[hand_arg >> 31], 1u);
+                if (lane == 0u) slot = atomicAdd(&handover[0], 1u);
                 slot = __builtin_amdgcn_readfirstlane(slot);
                 if (slot < kHandCap) {
                     if (lane == 0u) handover[kHandHeader + slot] = ((by * btiles_x + bx) << 2) | wv;
@@ -2369,7 +2377,7 @@ void launch(const DstParams &p, const DstAccelView &acc, const TileGrid &t, cons
             const uint32_t *block_order = nullptr, uint32_t *handover = nullptr, uint32_t hand_arg = 0u) {
     const uint32_t n_blocks = t.btiles_x * t.btiles_y;
     dim3 grid(n_blocks), block(kWavesPerBlock * DST_WAVE);
-    const bool takers = !BWD && handover != nullptr && (hand_arg & kHandStepsMask) == 0u;
+    const bool takers = !BWD && handover != nullptr && hand_arg == 0u;
     if (!BWD && kFwdWavesPerBlock == 1) {
         grid = dim3((n_blocks + 7u) / 8u * 32u);
         block = dim3(DST_WAVE);
@@ -2524,14 +2532,12 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
     } else {
         // the second launch of each pair traces the tiles the first one handed over (usually none: it leaves at once)
         uint32_t *const list = (kFwdWavesPerBlock == 1 && dst_handover_active(ctx)) ? ctx->handover : nullptr;
-        const uint32_t parity = (uint32_t)(ctx->handover_parity & 1u) << 31;
-        const uint32_t steps = std::min<uint32_t>(ctx->handover_steps, kHandStepsMask);
+        const uint32_t steps = std::max<uint32_t>(ctx->handover_steps, 1u);
         for (int pass = 0; pass < (list != nullptr ? 2 : 1); ++pass) {
-            const uint32_t arg = parity | (pass == 0 ? steps : 0u);
+            const uint32_t arg = pass == 0 ? steps : 0u;
             if (rec) launch<false, true>(p, acc, t, ray_order, stream, nullptr, list, arg);
             else launch<false, false>(p, acc, t, ray_order, stream, nullptr, list, arg);
         }
-        if (list != nullptr) ctx->handover_parity ^= 1u;
         if (det && p.training && p.a_weights != nullptr)
             hipLaunchKernelGGL(k_det_finish_weights, dim3(1024), dim3(256), 0, stream, p);
     }

@@ -226,7 +226,8 @@ int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_p
  * a context uses them only while its last build counted at least 2048 quads with edges below 1/2048 of the scene's
  * size (`small_quads`; refits do not recount); DST_HANDOVER_ALWAYS and DST_HANDOVER_OFF decide regardless of the
  * scene.  dst_set_handover: steps = 0 keeps the current limit.  DST_HANDOVER=off|auto|always and DST_HANDOVER_STEPS=n
- * in the environment of dst_create set the initial values.  dst_trace_info waits for the device; tiles_handed_over
+ * in the environment of dst_create set the initial values.  The list is emptied on the device by the second launch, so
+ * a forward call recorded into a graph can be replayed.  dst_trace_info waits for the device; tiles_handed_over
  * counts since the context was created (a 32-bit count). */
 #define DST_HANDOVER_OFF 0
 #define DST_HANDOVER_AUTO 1

@@ -200,6 +200,50 @@ def test_a_full_list_leaves_the_other_tiles_to_their_own_waves():
             assert np.array_equal(out[name].view(np.uint32), ref[name].view(np.uint32)), name
 
 
+def test_a_captured_forward_with_hand_over_can_be_replayed():
+    """Nothing on the host changes from one forward call to the next (the takers empty the list themselves), so the
+    launch pair can be recorded into a graph once and replayed: every replay hands the same tiles over and gives the
+    eager result, with eager work of the program between the replays."""
+    from diff_surfel_tracing import _C
+    sc = S.scene_cube(P=8000, seed=1)
+    o, d = S.rays_cube(64, 80)
+    g = {k: v.cuda() for k, v in sc.items()}
+    e, bg, eye = torch.empty(0, device="cuda"), torch.zeros(3, device="cuda"), torch.eye(4, device="cuda")
+    og, dg = o.cuda(), d.cuda()
+    tracer = own_tracer("off")
+    ctx = tracer.optix_context
+    tracer.build_acceleration_structure(g["vertices"], g["faces"], True)
+
+    def trace():
+        return _C.trace_surfels(ctx, False, True, og, dg, g["vertices"], bg, g["means3D"], g["shs"], 3, e, e,
+                                g["opacities"], g["scales"], 1.0, g["rotations"], e, eye, eye, bg, False, False, 0, 0.0)
+    ref = [t.clone() for t in trace()[:4]]
+    ctx.set_handover(_C.HANDOVER_ALWAYS, 40)
+    before = handed(tracer)
+    trace()
+    per_trace = handed(tracer) - before
+    assert per_trace > 10
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        trace()                                   # warm-up on a side stream, as torch asks before a capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = trace()
+    for k in range(4):
+        for t in out[:4]:
+            t.fill_(-7.0)
+        assert torch.isfinite(torch.randn(1000, device="cuda").sum()).item()   # eager work between the replays
+        before = handed(tracer)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert handed(tracer) - before == per_trace, k
+        for a, b in zip(out[:4], ref):
+            assert torch.equal(a, b), k
+
+
 def test_set_handover_rejects_unknown_modes():
     tracer = own_tracer("auto")
     with pytest.raises(RuntimeError):
