@@ -56,7 +56,7 @@ static_assert(sizeof(DstLeaf) == 96, "leaf records are 24 dwords");
 
 // Cheap conservative stand-in for the exact ray/quad test, one per leaf (same order): the quad as a parallelogram
 // on its mean plane.  A ray whose hit point on that plane has |s|, |r| beyond `lim0` (plus a margin for rounding)
-// cannot pass the exact test; the walk fetches the 80-byte record and runs the exact test only if some lane
+// cannot pass the exact test; the walk fetches the 96-byte record and runs the exact test only if some lane
 // survives.  c = centroid, n = unit normal, fu/fv = dual vectors of the averaged half edges (s = fu.(P-c),
 // r = fv.(P-c): the corners sit at about (+-1, +-1)), mfu = max(|fu|, |fv|), lim0 = largest |s| or |r| of a
 // corner, a little enlarged, tdev = how far the corners leave the mean plane, enlarged (0 for a planar quad),
