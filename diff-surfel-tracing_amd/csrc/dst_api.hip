@@ -189,6 +189,7 @@ int dst_trace_info(dst_ctx *ctx, DstTraceInfo *info) {
     info->handover_mode = (uint32_t)ctx->handover_mode;
     info->handover_steps = ctx->handover_steps;
     info->handover_capacity = kDstHandoverCap;
+    if (ctx->small_quads_asked && ctx->bounds_host) ctx->small_quads = ctx->bounds_host->small_quads;   // (the device is idle)
     info->small_quads = ctx->small_quads;
     info->handover_active = dst_handover_active(ctx) ? 1u : 0u;
     info->reserved = 0u;

@@ -75,7 +75,7 @@ struct DstBounds {          // device-resident reduction targets, order-preservi
     uint32_t max_depth;     // nodes above the deepest leaf (builds with two-level keys only)
     uint32_t scale;         // raw bits of a float: size of the scene's bulk (set by a build, kept by refits); what ray
                             // origins are compared with (packets, ray keys) - not a bound on anything
-    uint32_t small_quads;   // quads with edges below kDstSmallQuad of that size, counted by a build
+    uint32_t small_quads;   // quads with edges below kDstSmallQuad of that size, counted by every build and refit
 };
 // Quads this much smaller than the scene are smaller than a pixel at usual resolutions (a 1080p pixel at half the
 // scene's size away is about 5e-4 of it wide); a context whose last build counted kDstSmallQuadsMin of them traces
@@ -150,7 +150,9 @@ struct dst_ctx {
     uint32_t *handover = nullptr;      // device, behind `bounds`: kDstHandoverHeader words + kDstHandoverCap entries, zeroed at creation
     uint32_t handover_steps = kDstHandoverSteps;   // limit of a tile's first walk
     int handover_mode = DST_HANDOVER_AUTO;         // auto: only for scenes with many small quads
-    uint32_t small_quads = 0;          // as counted by the last build
+    uint32_t small_quads = 0;          // as counted by the last build, or by a refit since (see dst_launch_trace)
+    uint32_t small_quads_refits = 0;   // ctx->refits when the count was last asked for
+    bool small_quads_asked = false;    // a copy of the device's count into bounds_host has been enqueued since the build
     DstBounds *bounds = nullptr;       // device (allocated by dst_create together with the hand-over list)
     DstBounds *bounds_host = nullptr;  // pinned host copy
     void *core_box = nullptr;          // device: the box the two-level Morton keys are laid over (lbvh.hip)

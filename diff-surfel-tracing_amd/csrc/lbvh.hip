@@ -773,6 +773,23 @@ __global__ void k_fit_ranges(DstNode *nodes, RangeBoxes rb, uint32_t n_blocks, u
     }
 }
 
+// Is this quad far smaller than the scene (DstBounds::small_quads)?  `scale` = the scene's size as set by the last build.
+__device__ __forceinline__ bool quad_is_small(const float (&c)[4][3], float scale) {
+    float ab = 0.f, ac = 0.f;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        ab += (c[1][a] - c[0][a]) * (c[1][a] - c[0][a]);
+        ac += (c[2][a] - c[0][a]) * (c[2][a] - c[0][a]);
+    }
+    const float lim = scale * kDstSmallQuad;
+    return fmaxf(ab, ac) < lim * lim;
+}
+// One addition per wave that has any (scenes without small quads add nothing).
+__device__ __forceinline__ void count_small_quads(bool small, DstBounds *bounds) {
+    const unsigned long long m = __ballot(small);
+    if ((threadIdx.x & (DST_WAVE - 1)) == 0 && m != 0ull) atomicAdd(&bounds->small_quads, (uint32_t)__popcll(m));
+}
+
 // Leaf records in Morton order (also the whole of a refit's geometry update).
 __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__restrict__ quad_ids,
                             const uint32_t *__restrict__ sorted_ids, DstLeaf *__restrict__ leaves,
@@ -787,16 +804,7 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
         const uint32_t g = sorted_ids[i];
         load_corners(vertices, quad_ids[g], g, c);
         write_leaf(c, g, i, leaves, pre);
-        if (count_small != nullptr) {   // a build: quads far smaller than the scene (DstBounds::small_quads)
-            float ab = 0.f, ac = 0.f;
-#pragma unroll
-            for (int a = 0; a < 3; ++a) {
-                ab += (c[1][a] - c[0][a]) * (c[1][a] - c[0][a]);
-                ac += (c[2][a] - c[0][a]) * (c[2][a] - c[0][a]);
-            }
-            const float lim = __uint_as_float(count_small->scale) * kDstSmallQuad;
-            small = fmaxf(ab, ac) < lim * lim;
-        }
+        small = quad_is_small(c, __uint_as_float(count_small->scale));
 #pragma unroll
         for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -804,10 +812,7 @@ __global__ void k_leaf_fill(const float *__restrict__ vertices, const int4 *__re
     }
     if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
     if (bounds != nullptr) block_max_abs(mabs, bounds);   // a refit: the coordinate bound of the moved quads
-    if (count_small != nullptr) {
-        const unsigned long long m = __ballot(small);
-        if ((threadIdx.x & (DST_WAVE - 1)) == 0 && m != 0ull) atomicAdd(&count_small->small_quads, (uint32_t)__popcll(m));
-    }
+    count_small_quads(small, count_small);
 }
 
 // The same for a refit straight from the surfel parameters: the four corners of surfel g are
@@ -854,6 +859,7 @@ __global__ void k_leaf_fill_from_surfels(const float *__restrict__ means, const 
         }
         write_leaf(c, g, i, leaves, pre);
         }
+        count_small_quads(valid && quad_is_small(c, __uint_as_float(bounds->scale)), bounds);
         if (rb.lbox != nullptr) wave_range_boxes(c, valid, i, n, rb);
     }
     mabs = wave_max(mabs);
@@ -1317,7 +1323,7 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
     }
     if (surfels == nullptr)
         hipLaunchKernelGGL(k_leaf_fill, grid_for(n), dim3(kBlock), 0, stream, vertices, quad_ids, ctx->vals[0],
-                           ctx->leaves, ctx->pre, rb, rebuild ? nullptr : ctx->bounds, rebuild ? ctx->bounds : nullptr, n);
+                           ctx->leaves, ctx->pre, rb, rebuild ? nullptr : ctx->bounds, ctx->bounds, n);
     if (by_ranges) {
         const uint32_t n_blocks = (n + kRangeBlock - 1) / kRangeBlock;
         for (int level = 1; (2u << (level - 1)) <= n_blocks; ++level)
@@ -1356,6 +1362,8 @@ int dst_lbvh_build(dst_ctx *ctx, const float *vertices, uint32_t n_vertices, con
         }
         std::memcpy(&ctx->max_abs, &ctx->bounds_host->max_abs, 4);
         ctx->small_quads = ctx->bounds_host->small_quads;
+        ctx->small_quads_refits = ctx->refits;
+        ctx->small_quads_asked = false;
         if (ctx->fine_keys && ctx->bounds_host->max_depth > kMaxDepth) {
             // deeper than the walks' stacks are sized for (nested clusters at every scale): one-level keys, for good
             ctx->fine_keys = false;

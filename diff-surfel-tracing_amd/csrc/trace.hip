@@ -2530,6 +2530,17 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
             else hipLaunchKernelGGL(k_finish_grad_rows<8>, grid, block, 0, stream, p);
         }
     } else {
+        // Refits count the small quads too, on the device; the count comes over behind the first forward trace after
+        // a refit (a 4-byte copy on this stream, nobody waits for it) and serves the traces after that one.
+        if (ctx->bounds_host != nullptr && ctx->bounds != nullptr) {
+            if (ctx->small_quads_asked) ctx->small_quads = *(volatile const uint32_t *)&ctx->bounds_host->small_quads;
+            if (ctx->small_quads_refits != ctx->refits) {
+                DST_HIP(ctx, hipMemcpyAsync(&ctx->bounds_host->small_quads, &ctx->bounds->small_quads, sizeof(uint32_t),
+                                            hipMemcpyDeviceToHost, stream));
+                ctx->small_quads_refits = ctx->refits;
+                ctx->small_quads_asked = true;
+            }
+        }
         // the second launch of each pair traces the tiles the first one handed over (usually none: it leaves at once)
         uint32_t *const list = (kFwdWavesPerBlock == 1 && dst_handover_active(ctx)) ? ctx->handover : nullptr;
         const uint32_t steps = std::max<uint32_t>(ctx->handover_steps, 1u);

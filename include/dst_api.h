@@ -223,8 +223,9 @@ int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_p
  * ordinary scenes) is therefore put on a list and traced by a second launch in which every ray walks on its own: same
  * results bit for bit.  At most `handover_capacity` tiles per call are handed over; further ones are traced the usual
  * way.  The kernels that can hand over are 1 to 4 % slower than those that cannot, so by default (DST_HANDOVER_AUTO)
- * a context uses them only while its last build counted at least 2048 quads with edges below 1/2048 of the scene's
- * size (`small_quads`; refits do not recount); DST_HANDOVER_ALWAYS and DST_HANDOVER_OFF decide regardless of the
+ * a context uses them only while its last build or refit counted at least 2048 quads with edges below 1/2048 of the scene's
+ * size (`small_quads`; refits count too, and their count reaches the host behind the first forward trace that follows,
+ * so it serves from the second one on); DST_HANDOVER_ALWAYS and DST_HANDOVER_OFF decide regardless of the
  * scene.  dst_set_handover: steps = 0 keeps the current limit.  DST_HANDOVER=off|auto|always and DST_HANDOVER_STEPS=n
  * in the environment of dst_create set the initial values.  The list is emptied on the device by the second launch, so
  * a forward call recorded into a graph can be replayed.  dst_trace_info waits for the device; tiles_handed_over
@@ -234,7 +235,7 @@ int dst_accel_download(dst_ctx *ctx, void *nodes, void *leaves, uint32_t *node_p
 #define DST_HANDOVER_ALWAYS 2
 typedef struct DstTraceInfo {
     uint32_t handover_mode, handover_steps, handover_capacity;
-    uint32_t small_quads;        /* as counted by the last build */
+    uint32_t small_quads;        /* as counted by the last build, or by a refit whose count has arrived */
     uint32_t handover_active;    /* 1: the next forward trace uses the kernels that can hand tiles over */
     uint32_t reserved;
     uint64_t tiles_handed_over;

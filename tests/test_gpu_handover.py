@@ -244,6 +244,30 @@ def test_a_captured_forward_with_hand_over_can_be_replayed():
             assert torch.equal(a, b), k
 
 
+def test_refits_recount_the_small_quads():
+    """A structure built over ordinary quads and refitted to quads a thousand times smaller (and back): the count
+    made by the refit arrives behind the first forward trace after it and switches the hand-over for the next ones."""
+    tracer = own_tracer("auto")
+    ctx = tracer.optix_context
+    sc = S.scene_cube(P=9000, seed=2)
+    o, d = S.rays_cube(32, 32)
+    gpu_trace(tracer, sc, o, d, training=False)
+    assert (ctx.trace_info().small_quads, ctx.trace_info().handover_active) == (0, 0)
+    for shrink, want in ((1e-3, 8000), (1.0, 0)):
+        moved = dict(sc)
+        moved["scales"] = (sc["scales"] * shrink).contiguous()
+        if shrink < 1.0:     # from the surfel parameters
+            moved["vertices"] = tracer.refit_from_surfels(moved["means3D"].cuda(), moved["scales"].cuda(),
+                                                          moved["rotations"].cuda()).cpu()
+        else:                # from a vertex buffer
+            moved["vertices"], _ = S.get_triangles(moved["means3D"], moved["scales"], moved["rotations"])
+            tracer.build_acceleration_structure(moved["vertices"].cuda(), sc["faces"].cuda(), False)
+        gpu_trace(tracer, moved, o, d, training=False, build=False)
+        info = ctx.trace_info()
+        assert (info.small_quads >= want if want else info.small_quads == 0), (shrink, info.small_quads)
+        assert info.handover_active == (1 if want else 0)
+
+
 def test_set_handover_rejects_unknown_modes():
     tracer = own_tracer("auto")
     with pytest.raises(RuntimeError):
