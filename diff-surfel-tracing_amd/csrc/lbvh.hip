@@ -937,11 +937,19 @@ __global__ __launch_bounds__(kFitBlock) void k_fit(DstNode *nodes, const uint32_
 
 // Reference the trace kernels follow for a child of a binary node: a subtree of at most DST_GROUP leaves
 // (contiguous in Morton order) is one leaf group, anything larger is the wide node of the same index.
-__device__ __forceinline__ uint32_t traversal_ref(const DstNode *__restrict__ nodes, uint32_t c) {
+// The child's leaves first .. last are known from its parent (first .. split and split + 1 .. last): no look at the
+// child's own record.
+__device__ __forceinline__ uint32_t traversal_ref(uint32_t c, uint32_t first, uint32_t last) {
     if (c & DST_LEAF_BIT) return DST_LEAF_BIT | (c & DST_REF_FIRST_MASK);
-    const uint32_t first = nodes[c].first, count = nodes[c].last - first + 1u;
+    const uint32_t count = last - first + 1u;
     if (count <= DST_GROUP) return DST_LEAF_BIT | ((count - 1u) << 28) | first;
     return c;
+}
+// Both children of a node as traversal references.
+__device__ __forceinline__ void child_refs(const DstNode &nd, uint32_t &r0, uint32_t &r1) {
+    const uint32_t split = nd.c0 & ~DST_LEAF_BIT;
+    r0 = traversal_ref(nd.c0, nd.first, split);
+    r1 = traversal_ref(nd.c1, split + 1u, nd.last);
 }
 
 // Collapse the fitted binary hierarchy into 4-wide traversal nodes.  Two ways: node i offers its grandchildren (a child
@@ -967,18 +975,21 @@ __global__ void k_widen(const DstNode *__restrict__ nodes, DstWideNode *__restri
         w.ref[k] = ref;
         ++k;
     };
+    uint32_t own[2];
+    child_refs(nd, own[0], own[1]);
     if (!by_area) {
-        const uint32_t cs[2] = {nd.c0, nd.c1};
         const float *los[2] = {nd.lo0, nd.lo1}, *his[2] = {nd.hi0, nd.hi1};
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            const uint32_t r = traversal_ref(nodes, cs[s]);
+            const uint32_t r = own[s];
             if (r & DST_LEAF_BIT) {
                 put(los[s], his[s], r);
             } else {
-                const DstNode ch = nodes[cs[s]];
-                put(ch.lo0, ch.hi0, traversal_ref(nodes, ch.c0));
-                put(ch.lo1, ch.hi1, traversal_ref(nodes, ch.c1));
+                const DstNode ch = nodes[r];
+                uint32_t g0, g1;
+                child_refs(ch, g0, g1);
+                put(ch.lo0, ch.hi0, g0);
+                put(ch.lo1, ch.hi1, g1);
             }
         }
     } else {
@@ -990,8 +1001,8 @@ __global__ void k_widen(const DstNode *__restrict__ nodes, DstWideNode *__restri
             lo[0][a] = nd.lo0[a]; hi[0][a] = nd.hi0[a];
             lo[1][a] = nd.lo1[a]; hi[1][a] = nd.hi1[a];
         }
-        ref[0] = traversal_ref(nodes, nd.c0);
-        ref[1] = traversal_ref(nodes, nd.c1);
+        ref[0] = own[0];
+        ref[1] = own[1];
         while (m < DST_WIDE) {
             int best = -1;
             float best_area = -1.f;
@@ -1020,8 +1031,7 @@ __global__ void k_widen(const DstNode *__restrict__ nodes, DstWideNode *__restri
                 lo[best][a] = ch.lo0[a]; hi[best][a] = ch.hi0[a];
                 lo[best + 1][a] = ch.lo1[a]; hi[best + 1][a] = ch.hi1[a];
             }
-            ref[best] = traversal_ref(nodes, ch.c0);
-            ref[best + 1] = traversal_ref(nodes, ch.c1);
+            child_refs(ch, ref[best], ref[best + 1]);
             ++m;
         }
         for (int c = 0; c < m; ++c) put(lo[c], hi[c], ref[c]);
