@@ -109,6 +109,11 @@ typedef struct DstParams {
      * atomics make a_weights and the per-surfel gradients depend on the order in which rays finish): every
      * atomically accumulated sum is formed in 64-bit fixed point, where addition is exact and hence independent of
      * order, in this buffer, and converted to fp32 into the caller's tensor by a closing kernel of the same call.
+     * Range: the gradients of scales, rotations, means and the densification gradient are kept in units of 2^-36 and
+     * hold sums up to about 6.7e7 in magnitude, everything else (colours, SH, opacity, aux, a_weights) in units of
+     * 2^-40 up to about 4.2e6; an addend beyond the range is clamped to it and sums beyond it wrap.  Losses whose
+     * per-surfel gradients can get there (coordinates in the tens of kilometres with upstream gradients of order
+     * one) have to be scaled down by the caller, or traced without this flag.
      * Device memory, dst_det_workspace_words() 8-byte words, zero-filled by the caller before each call. */
     unsigned long long *det_workspace;
     /* optional gradient rows (no counterpart in the reference): dst_det_workspace_words(P, aux, 1) floats of device

@@ -164,6 +164,9 @@ def test_random_configuration(oracle, tracer, case):
     if depth > 0:
         kw.update(max_trace_depth=depth, specular_threshold=float(rng.choice([0.0, 0.1, 0.4])))
     grads = True
+    if mode == "det" and trait == "huge":
+        # gradients of a 30 km scene reach 1e9, beyond the fixed range of the deterministic sums (include/dst_api.h)
+        mode = "plain"
     if trait == "outliers":
         # its builds go over to two-level keys for good: a context of its own, the session's keeps its one-level keys
         import diff_surfel_tracing as dst
