@@ -192,7 +192,7 @@ int dst_trace_info(dst_ctx *ctx, DstTraceInfo *info) {
     if (ctx->small_quads_asked && ctx->bounds_host) ctx->small_quads = ctx->bounds_host->small_quads;   // (the device is idle)
     info->small_quads = ctx->small_quads;
     info->handover_active = dst_handover_active(ctx) ? 1u : 0u;
-    info->reserved = 0u;
+    info->det_out_of_range = words[kDstHandoverOutOfRange];
     info->tiles_handed_over = words[2];
     return DST_OK;
 }

@@ -97,6 +97,7 @@ struct DstAccelView {
 // Tile hand-over list of the forward trace (layout: trace.hip).  Steps: walks of the benchmark scenes take a few
 // hundred; DST_HANDOVER_STEPS in the environment of dst_create sets another limit.
 constexpr uint32_t kDstHandoverHeader = 4, kDstHandoverCap = 8192, kDstHandoverSteps = 2048;
+constexpr uint32_t kDstHandoverOutOfRange = 3;   // header word lent to the deterministic mode's out-of-range count
 // The list shares its allocation with the bounds (made by dst_create).
 constexpr size_t kDstHandoverOffset = 64;   // bytes from the bounds to the list
 static_assert(sizeof(DstBounds) <= kDstHandoverOffset, "the hand-over list starts behind the bounds");

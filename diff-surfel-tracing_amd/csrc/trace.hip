@@ -936,8 +936,10 @@ template <int AUXM, bool DET> struct TableRows {
 // Integer addition is exact, so a sum of fixed-point numbers does not depend on the order of its terms: every
 // atomically accumulated value (LDS table, global memory) is converted first.  2^-36 units for the geometric
 // columns (scale, rotation, mean, densification: range +-6.7e7), 2^-40 for the others and for the blending
-// weights (+-4.2e6); a value outside the range saturates.
+// weights (+-4.2e6); a value outside the range saturates.  The closing kernels count the sums they find in the outer
+// half of the range (one saturated term puts a sum there), so that a scene too large for the mode is noticed.
 constexpr int kDetShiftGeo = 36, kDetShiftOther = 40;
+__device__ __forceinline__ bool det_out_of_range(long long q) { return q >= (1LL << 61) || q <= -(1LL << 61); }
 __device__ __forceinline__ int det_shift(int col) { return (col >= kColScale && col < kColSh) ? kDetShiftGeo : kDetShiftOther; }
 __device__ __forceinline__ long long to_fixed(float v, int shift) {
     float x = __builtin_ldexpf(v, shift);                       // exact scaling
@@ -1908,8 +1910,8 @@ __global__ __launch_bounds__(1024) void k_block_order(const uint32_t *__restrict
 // own - the same buffer content, so the same results bit for bit.  List: word 0 = tiles listed by this trace, word 1 =
 // takers that have read their entry (the last one empties the list for the next trace: nothing on the host changes
 // from call to call, so a captured launch pair can be replayed), word 2 = tiles handed over since the context was
-// made, entries ((by * btiles_x + bx) * 4 + wave) from word 4.  A wave that finds the list full starts again without
-// a limit.
+// made, word 3 = not the list's: sums of the deterministic mode found out of range (its closing kernels count there),
+// entries ((by * btiles_x + bx) * 4 + wave) from word 4.  A wave that finds the list full starts again without a limit.
 constexpr uint32_t kHandHeader = kDstHandoverHeader, kHandCap = kDstHandoverCap;
 template <bool BWD, int AUXM, bool REC, bool MIXED, bool DET, bool HAND>
 __device__ __forceinline__ void trace_body(const DstParams &p, const DstAccelView &acc, int tw_log2, int th_log2,
@@ -2264,12 +2266,13 @@ void k_trace_bwd(const DstParams p, const DstAccelView acc, int tw_log2, int th_
 
 // Closing kernels of the deterministic mode: fixed point -> fp32, added to the caller's (zero-filled) tensors.
 template <int AUXM>
-__global__ void k_det_finish_grads(const DstParams p) {
+__global__ void k_det_finish_grads(const DstParams p, uint32_t *out_of_range) {
     constexpr int cols = RowLayout<AUXM>::cols;
     const size_t n = (size_t)p.P * cols;
     for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < n; k += (size_t)gridDim.x * blockDim.x) {
         const long long q = (long long)p.det_workspace[k];
         if (q == 0) continue;
+        if (det_out_of_range(q)) atomicAdd(out_of_range, 1u);
         const uint32_t g = (uint32_t)(k / cols);
         const int col = (int)(k - (size_t)g * cols);
         float *dst = tensor_address<AUXM>(p, g, col);
@@ -2290,10 +2293,11 @@ __global__ void k_finish_grad_rows(const DstParams p) {
         if (dst != nullptr) *dst += v;
     }
 }
-__global__ void k_det_finish_weights(const DstParams p) {
+__global__ void k_det_finish_weights(const DstParams p, uint32_t *out_of_range) {
     for (int g = blockIdx.x * blockDim.x + threadIdx.x; g < p.P; g += gridDim.x * blockDim.x) {
         const long long q = (long long)p.det_workspace[g];
         if (q != 0) p.a_weights[g] += from_fixed(q, kDetShiftOther);
+        if (det_out_of_range(q)) atomicAdd(out_of_range, 1u);
     }
 }
 
@@ -2499,6 +2503,7 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
     acc.root = dst_root_ref(ctx->n_leaves);
     const bool rec = p.hit_record != nullptr;
     const bool det = (p.flags & DST_FLAG_DETERMINISTIC) != 0u;
+    uint32_t *const out_of_range = ctx->handover + kDstHandoverOutOfRange;   // (a spare word of the list's header)
     if (backward) {
         const uint32_t n_blocks = t.btiles_x * t.btiles_y;
         if (rec && n_blocks < kOrderMinBlocks) {
@@ -2521,9 +2526,9 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
         launch<true, false>(p, acc, t, ray_order, stream);           // else this one does (it returns at once otherwise)
         const dim3 grid(2048), block(256);
         if (det) {
-            if (p.aux <= 2) hipLaunchKernelGGL(k_det_finish_grads<2>, grid, block, 0, stream, p);
-            else if (p.aux <= 4) hipLaunchKernelGGL(k_det_finish_grads<4>, grid, block, 0, stream, p);
-            else hipLaunchKernelGGL(k_det_finish_grads<8>, grid, block, 0, stream, p);
+            if (p.aux <= 2) hipLaunchKernelGGL(k_det_finish_grads<2>, grid, block, 0, stream, p, out_of_range);
+            else if (p.aux <= 4) hipLaunchKernelGGL(k_det_finish_grads<4>, grid, block, 0, stream, p, out_of_range);
+            else hipLaunchKernelGGL(k_det_finish_grads<8>, grid, block, 0, stream, p, out_of_range);
         } else if (p.grad_rows != nullptr) {
             if (p.aux <= 2) hipLaunchKernelGGL(k_finish_grad_rows<2>, grid, block, 0, stream, p);
             else if (p.aux <= 4) hipLaunchKernelGGL(k_finish_grad_rows<4>, grid, block, 0, stream, p);
@@ -2550,7 +2555,7 @@ int dst_launch_trace(dst_ctx *ctx, const DstParams &p_in, bool backward, hipStre
             else launch<false, false>(p, acc, t, ray_order, stream, nullptr, list, arg);
         }
         if (det && p.training && p.a_weights != nullptr)
-            hipLaunchKernelGGL(k_det_finish_weights, dim3(1024), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL(k_det_finish_weights, dim3(1024), dim3(256), 0, stream, p, out_of_range);
     }
     DST_HIP(ctx, hipGetLastError());
     return DST_OK;

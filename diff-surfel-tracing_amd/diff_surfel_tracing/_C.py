@@ -51,7 +51,7 @@ class DstAccelInfo(C.Structure):
 
 class DstTraceInfo(C.Structure):
     _fields_ = [("handover_mode", C.c_uint32), ("handover_steps", C.c_uint32), ("handover_capacity", C.c_uint32),
-                ("small_quads", C.c_uint32), ("handover_active", C.c_uint32), ("reserved", C.c_uint32),
+                ("small_quads", C.c_uint32), ("handover_active", C.c_uint32), ("det_out_of_range", C.c_uint32),
                 ("tiles_handed_over", C.c_uint64)]
 
 
@@ -217,6 +217,8 @@ class OptiXStateWrapper:
         self.records_skipped = 0            # forward calls that made no record because of the two limits above
         self.record_wanted = True           # set by the autograd wrapper for the call that follows
         self.deterministic = False          # True: a_weights and per-surfel gradients are bitwise reproducible
+        self.deterministic_check = True     # with `deterministic`: warn after a backward trace whose sums left the range
+        self._det_out_of_range = 0          # the library's count when last looked at
         self.gradient_rows = True           # backward sums per-surfel gradients in one row per surfel first (faster)
         self.distortion = False             # True: the dist output carries the 2DGS depth distortion (else zeros)
         self.sh_half = False                # True: the traces read the SH coefficients from a binary16 copy
@@ -315,10 +317,22 @@ class OptiXStateWrapper:
 
     def trace_info(self):
         """Tile hand-over of the forward trace (include/dst_api.h): mode, step limit, list capacity, the small quads the
-        last build counted, whether the next forward trace can hand over, tiles handed over so far.  Waits."""
+        last build counted, whether the next forward trace can hand over, tiles handed over so far; and the number of
+        sums the deterministic mode has found out of its fixed-point range.  Waits."""
         info = DstTraceInfo()
         _check(self, load_library().dst_trace_info(self.handle, C.byref(info)))
         return info
+
+    def check_deterministic_range(self):
+        """Warn if sums of the deterministic mode have left their fixed-point range since the last look (gradients
+        beyond about 6.7e7 for scales, rotations and means, 4.2e6 for the rest: they come out clamped or wrapped).
+        Waits for the device.  Returns the number of such sums."""
+        seen = int(self.trace_info().det_out_of_range)
+        new, self._det_out_of_range = (seen - self._det_out_of_range) & 0xFFFFFFFF, seen
+        if new:
+            warnings.warn("deterministic mode: %d per-surfel sums left the fixed-point range and are wrong; scale the "
+                          "loss down or trace without the mode" % new, RuntimeWarning, stacklevel=3)
+        return new
 
     def set_handover(self, mode, steps=0):
         """HANDOVER_OFF / HANDOVER_AUTO (only for scenes with many quads far smaller than the scene) / HANDOVER_ALWAYS;
@@ -527,6 +541,8 @@ def trace_surfels_backward(ctx, start_from_first, ray_o, ray_d, vertices, backgr
     _check(ctx, load_library().dst_trace_backward(ctx.handle, C.byref(p), _stream()))
     if events is not None:
         events[1].record()
+    if p.flags & FLAG_DETERMINISTIC and getattr(ctx, "deterministic_check", False):
+        ctx.check_deterministic_range()   # (the mode waits for the device elsewhere too: record sizes)
     del keep
     return (dL_dray_o, dL_dray_d, dL_dmeans3D, dL_dgrads3D, dL_dgrads3D_abs, dL_dshs, dL_dcolors, dL_dothers,
             dL_dopacities, dL_dscales, dL_drotations, dL_dtransMat)

@@ -113,7 +113,9 @@ typedef struct DstParams {
      * hold sums up to about 6.7e7 in magnitude, everything else (colours, SH, opacity, aux, a_weights) in units of
      * 2^-40 up to about 4.2e6; an addend beyond the range is clamped to it and sums beyond it wrap.  Losses whose
      * per-surfel gradients can get there (coordinates in the tens of kilometres with upstream gradients of order
-     * one) have to be scaled down by the caller, or traced without this flag.
+     * one) have to be scaled down by the caller, or traced without this flag.  The closing kernel counts the sums
+     * it finds in the outer half of the range (one clamped addend puts a sum there; a sum that wrapped all the way
+     * into the inner half escapes the count): DstTraceInfo.det_out_of_range, 0 as long as every sum was in range.
      * Device memory, dst_det_workspace_words() 8-byte words, zero-filled by the caller before each call. */
     unsigned long long *det_workspace;
     /* optional gradient rows (no counterpart in the reference): dst_det_workspace_words(P, aux, 1) floats of device
@@ -242,7 +244,7 @@ typedef struct DstTraceInfo {
     uint32_t handover_mode, handover_steps, handover_capacity;
     uint32_t small_quads;        /* as counted by the last build, or by a refit whose count has arrived */
     uint32_t handover_active;    /* 1: the next forward trace uses the kernels that can hand tiles over */
-    uint32_t reserved;
+    uint32_t det_out_of_range;   /* DST_FLAG_DETERMINISTIC: sums found in the outer half of their range since dst_create */
     uint64_t tiles_handed_over;
 } DstTraceInfo;
 int dst_trace_info(dst_ctx *ctx, DstTraceInfo *info);

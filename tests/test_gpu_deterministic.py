@@ -89,3 +89,37 @@ def test_the_c_abi_rejects_the_flag_without_a_workspace(tracer):
     p.flags = binding.FLAG_DETERMINISTIC
     rc = lib.dst_trace_forward(tracer.optix_context.handle, C.byref(p), None)
     assert rc == 1 and b"det_workspace" in lib.dst_last_error(tracer.optix_context.handle)
+
+
+def test_sums_beyond_the_fixed_point_range_are_counted_and_warned_about(tracer):
+    """Per-surfel gradients beyond about 6.7e7 (4.2e6 for colours and opacity) do not fit the mode's 64-bit fixed
+    point: the closing kernel counts them and the binding warns after the backward trace; gradients of ordinary
+    size are not counted."""
+    import warnings
+    sc = S.scene_cube(P=2000, seed=3)
+    o, d = S.rays_cube(64, 64)
+    ug = upstream(o.shape[0], o.shape[1], 2)
+    huge = {k: v * 1e12 for k, v in ug.items()}
+    ctx = tracer.optix_context
+    tracer.deterministic = True
+    try:
+        ctx.check_deterministic_range()                # (whatever earlier tests left)
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            _run(tracer, sc, o, d, ug)
+        assert ctx.check_deterministic_range() == 0
+        with pytest.warns(RuntimeWarning, match="left the fixed-point range"):
+            _run(tracer, sc, o, d, huge)
+        before = ctx.trace_info().det_out_of_range
+        assert before > 0
+        ctx.deterministic_check = False                # the count goes on, the warning does not
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            _run(tracer, sc, o, d, huge)
+        assert ctx.trace_info().det_out_of_range > before
+    finally:
+        ctx.deterministic_check = True
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            ctx.check_deterministic_range()
+        tracer.deterministic = False
