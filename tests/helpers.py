@@ -108,7 +108,10 @@ def _noise_rules(name, err, base, extra, ref_abs, max_noisy, finite):
     loud = np.zeros_like(noisy) if np.isscalar(extra) else ((extra > LOUD_NOISE * ref_abs) & (ref_abs > base) & finite)
     NOISE_LOG.append((name, int(noisy.size), int(noisy.sum()), int(loud.sum())))
     assert noisy.sum() <= max(max_noisy * noisy.size, MIN_NOISY), (
-        "%s: %d of %d elements (%.3g) pass only through the noise allowance" % (name, noisy.sum(), noisy.size, noisy.mean()))
+        "%s: %d of %d elements (%.3g) pass only through the noise allowance; they miss the plain bound by factors of %s, "
+        "relative errors %s" % (name, noisy.sum(), noisy.size, noisy.mean(),
+                                np.round(np.sort((err / np.maximum(base, 1e-300))[noisy])[-8:], 2).tolist(),
+                                ["%.2g" % x for x in np.sort((err / np.maximum(ref_abs, 1e-300))[noisy])[-8:]]))
     assert loud.sum() <= max(MAX_LOUD * loud.size, MIN_NOISY), (
         "%s: the noise allowance alone exceeds %.0f %% of the value on %d of %d elements" % (
             name, 100 * LOUD_NOISE, loud.sum(), loud.size))

@@ -10,6 +10,7 @@ surfel parameters).  Drawn from generators of their own, so that the cases above
 tile hand-over forced to 1 or to 48 steps in half of them.  The cases are small; their value is in the combinations no
 hand-written test makes."""
 import os
+import warnings
 
 import numpy as np
 import pytest
@@ -164,9 +165,6 @@ def test_random_configuration(oracle, tracer, case):
     if depth > 0:
         kw.update(max_trace_depth=depth, specular_threshold=float(rng.choice([0.0, 0.1, 0.4])))
     grads = True
-    if mode == "det" and trait == "huge":
-        # gradients of a 30 km scene reach 1e9, beyond the fixed range of the deterministic sums (include/dst_api.h)
-        mode = "plain"
     if trait == "outliers":
         # its builds go over to two-level keys for good: a context of its own, the session's keeps its one-level keys
         import diff_surfel_tracing as dst
@@ -179,20 +177,36 @@ def test_random_configuration(oracle, tracer, case):
         # as it is, and ten times the packet walk's time with every ray walking on its own
         hand = "auto"
     import helpers
-    shares = (helpers.MAX_LOUD, helpers.MAX_NOISY)
+    shares = (helpers.MAX_LOUD, helpers.MAX_NOISY, helpers.MIN_NOISY)
     try:
         if hand != "auto":
             ctx.set_handover(2, int(hand.split("_")[1]))
         # The shares of elements that may lean on the rounding allowance are set for the benchmark scenes.  Here the
         # traits make ill-conditioned gradients the rule (a surfel of a tenth of a millimetre, a scene 3 km from the
         # origin: the hit point is known to 1e-7 of its distance, whoever computes it), so many elements carry a wide
-        # allowance; the element-wise bound itself is the same as everywhere.
-        helpers.MAX_LOUD, helpers.MAX_NOISY = 1.0, 2e-2
+        # allowance; the element-wise bound itself is the same as everywhere.  Eight elements of a small tensor may
+        # lean on it: forty surfels far larger than their scene and stretched 25:1 had six of their eighty scale
+        # gradients there (sums that cancel to a hundredth of their terms: the oracle in float is 2.6 % from the oracle
+        # in double on the worst of them, the GPU 0.4 %).
+        helpers.MAX_LOUD, helpers.MAX_NOISY, helpers.MIN_NOISY = 1.0, 2e-2, 8
         if mode == "det":
             tracer.deterministic = True
-            check_case(oracle, tracer, sc, o, d, grads=grads, **kw)               # sizes the record
-            a, _ = check_case(oracle, tracer, sc, o, d, grads=grads, **kw)
-            b, _ = check_case(oracle, tracer, sc, o, d, grads=grads, **kw)
+            ctx.check_deterministic_range()                                       # (whatever earlier cases left)
+            with warnings.catch_warnings(record=True) as caught:
+                warnings.simplefilter("always")
+                try:
+                    check_case(oracle, tracer, sc, o, d, grads=grads, **kw)       # sizes the record
+                    a, _ = check_case(oracle, tracer, sc, o, d, grads=grads, **kw)
+                    b, _ = check_case(oracle, tracer, sc, o, d, grads=grads, **kw)
+                except AssertionError:
+                    # gradients beyond the mode's fixed range (a 0.1 mm scene of surfels 30 times smaller still: 7.7e7
+                    # on a mean; a 30 km scene: 1e9) come out clamped, and the binding has to have said so; such a scene is traced without
+                    # the mode, as the warning advises
+                    if not any("left the fixed-point range" in str(w.message) for w in caught):
+                        raise
+                    a = b = {}
+                    tracer.deterministic = False
+                    check_case(oracle, tracer, sc, o, d, grads=grads, **kw)
             for k, v in (a.get("grads_gpu") or {}).items():
                 if v is not None:
                     assert np.array_equal(v.view(np.uint32), b["grads_gpu"][k].view(np.uint32)), k
@@ -220,4 +234,4 @@ def test_random_configuration(oracle, tracer, case):
         tracer.deterministic = False
         ctx.record_max_bytes, ctx.gradient_rows = saved
         ctx.set_handover(1, 2048)
-        helpers.MAX_LOUD, helpers.MAX_NOISY = shares
+        helpers.MAX_LOUD, helpers.MAX_NOISY, helpers.MIN_NOISY = shares
