@@ -137,7 +137,7 @@ class _Rebuilding:
             self._tracer.build_acceleration_structure(v, f, False)
 
 
-N_CASES = int(os.environ.get("DST_SWEEP_CASES", "36"))   # more on demand (7900 pass)
+N_CASES = int(os.environ.get("DST_SWEEP_CASES", "36"))   # more on demand (10 800 pass)
 FIRST_CASE = int(os.environ.get("DST_SWEEP_FIRST", "5000"))
 
 
